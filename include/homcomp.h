@@ -1,0 +1,113 @@
+/*
+ * homcomp.h -- C ABI of the MI355X HomComp library (libhomcomp_amd.so).
+ *
+ * HomComp is an error-bounded lossy codec for float32 with a homomorphic sum: two compressed
+ * streams (or a stream and raw data) are added in the quantised-integer domain and re-encoded
+ * without dequantising.  Each entry point names the reference interface it replaces (paths are
+ * relative to the reference repository's HomComp/ directory).
+ *
+ * Conventions
+ *   - All data pointers are device pointers on the device that was current when the workspace
+ *     was created.  float / int32 buffers must be 16-byte aligned; stream buffers may have any
+ *     alignment.  Input and output buffers must not overlap.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued
+ *     asynchronously; nothing blocks except homcomp_last_size().
+ *   - `eb` is always an ABSOLUTE error bound (> 0).  Value-range-relative bounds are turned into
+ *     absolute ones with homcomp_range_f32() + homcomp_rel_to_abs().
+ *   - A stream of nbEle elements is  header[homcomp_header_bytes(nbEle)] || payload  and can take
+ *     up to homcomp_max_stream_bytes(nbEle) bytes; every output stream buffer needs that
+ *     capacity.  nbEle may be any count; elements past nbEle up to the next multiple of 32768
+ *     are encoded as zeros (what the reference sees in a zero-padded buffer).
+ *   - Sizes reported are TRUE stream lengths L.  The reference's wrappers report L +
+ *     header_bytes (src/GSZ_entry.cu:291-295 adds the header twice); homcomp_ref_cmpsize()
+ *     gives that number.
+ *   - A workspace holds the scan state of one call at a time: calls sharing a workspace must be
+ *     ordered on one stream (or otherwise serialised).  Use one workspace per concurrent stream.
+ *   - Every function returns HOMCOMP_OK (0) or a negative HOMCOMP_ERR_* code; no call aborts.
+ */
+#ifndef HOMCOMP_H
+#define HOMCOMP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HOMCOMP_OK 0
+#define HOMCOMP_ERR_INVALID_ARG (-1)  /* NULL pointer, eb <= 0 or not finite                   */
+#define HOMCOMP_ERR_ALIGNMENT (-2)    /* float / int32 buffer not 16-byte aligned               */
+#define HOMCOMP_ERR_TOO_LARGE (-3)    /* nbEle exceeds the workspace's max_nbEle                */
+#define HOMCOMP_ERR_HIP (-4)          /* a HIP runtime call failed; see homcomp_last_hip_error  */
+#define HOMCOMP_ERR_NO_DEVICE (-5)    /* no usable GPU                                           */
+
+typedef struct homcomp_workspace homcomp_workspace;
+
+const char *homcomp_status_string(int status);
+/* hipError_t of the most recent failing HIP call on this thread (0 if none). */
+int homcomp_last_hip_error(void);
+
+/* rate_ofs of src/GSZ.cu:48-50: one header byte per 32-element block of the padded length. */
+size_t homcomp_header_bytes(size_t nbEle);
+/* Worst-case stream length: header + 128 payload bytes per block.  (The reference allocates
+ * only 4*nbEle, src/homcomp_eval.cu:176, which incompressible input can overrun.) */
+size_t homcomp_max_stream_bytes(size_t nbEle);
+/* The value the reference's wrappers store in *cmpSize for a stream of true length L. */
+size_t homcomp_ref_cmpsize(size_t stream_len, size_t nbEle);
+
+/* Replaces the per-call cudaMalloc/cudaMemset/cudaFree of three (codec) or six (homomorphic
+ * sum) scratch arrays in src/GSZ_entry.cu:275-280,519-530 -- the shape
+ * allreduce_ring_comprs_hom_sum_F_opt hoists out of its loop (src/cuda_awareallreduce.cu:745-760). */
+int homcomp_workspace_create(homcomp_workspace **ws, size_t max_nbEle);
+int homcomp_workspace_destroy(homcomp_workspace *ws);
+
+/* GSZ_compress_deviceptr_outlier (include/GSZ_entry.h:14-16, src/GSZ_entry.cu:263-301).
+ * d_stream_len (optional, device uint64) receives L when the kernel finishes. */
+int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float eb,
+                         unsigned char *d_cmp, uint64_t *d_stream_len, void *stream);
+
+/* GSZ_decompress_deviceptr_outlier (include/GSZ_entry.h:17-20, src/GSZ_entry.cu:317-350).
+ * Blocks whose payload starts at or beyond cmp_size are skipped (src/GSZ.cu:908-911).  Skipped
+ * and rate-0 blocks are written as 0.0f (the reference leaves them untouched; identical on a
+ * pre-zeroed buffer). */
+int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
+                           size_t nbEle, float eb, float *d_out, void *stream);
+
+/* homomorphic_sum_F (include/GSZ_entry.h:33-36, src/GSZ_entry.cu:504-550): out = encode(
+ * deltas(in) + Lorenzo(quantise(local))). */
+int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
+                        const float *d_local, size_t nbEle, float eb, unsigned char *d_cmp_out,
+                        uint64_t *d_stream_len, void *stream);
+
+/* homomorphic_sum (include/GSZ_entry.h:29-32, src/GSZ_entry.cu:456-502): the local operand is the
+ * int32 output of homcomp_quant_predict_f32. */
+int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
+                        const int32_t *d_local_delta, size_t nbEle, unsigned char *d_cmp_out,
+                        uint64_t *d_stream_len, void *stream);
+
+/* Stream (+) stream: the combine stage of src/homcomp.cu:3611-3616 with both operands decoded
+ * from streams.  Equals homcomp_hom_sum_f32(a, x) when b = compress(x) with the same eb. */
+int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t size_a,
+                    const unsigned char *d_cmp_b, size_t size_b, size_t nbEle,
+                    unsigned char *d_cmp_out, uint64_t *d_stream_len, void *stream);
+
+/* kernel_quant_prediction (include/homcomp.cuh:2-5, src/homcomp.cu:1553-1602), which callers of
+ * the reference launch directly.  Writes nbEle int32 deltas. */
+int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,
+                              void *stream);
+
+/* The min/max scan of src/homcomp_eval.cu:156-163, on the device.  d_minmax: device float[2]. */
+int homcomp_range_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float *d_minmax,
+                      void *stream);
+/* src/homcomp_eval.cu:165: eb_abs = fl(rel * fl(max - min)) in float32 (host arithmetic). */
+float homcomp_rel_to_abs(float rel, float vmin, float vmax);
+
+/* The blocking read-back of src/GSZ_entry.cu:291 (cudaMemcpy of cmpOffset[gsize-1]): waits for
+ * `stream` and returns the length L produced by the last stream-producing call on ws. */
+int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HOMCOMP_H */

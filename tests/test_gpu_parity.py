@@ -1,0 +1,262 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on the same seeded inputs.
+
+Bar: byte-exact streams (header bytes, payload, length), bit-exact decompressed floats and
+quantised integers.  Floating-point bound checks use |x - x'| <= eb + 2^-21 * |x| (float32
+rounding of x/2eb and of q*eb*2 can add up to ~1.2 eb-relative slack at eb = 1e-6).
+"""
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, first_diff
+
+pytestmark = pytest.mark.gpu
+
+MAX_N = 1 << 22
+
+
+@pytest.fixture(scope="module")
+def gpu(pkg, cuda):
+    g = Gpu(pkg, cuda, MAX_N)
+    yield g
+    g.close()
+
+
+def make(gen, kind, n, seed=1):
+    return gen.GENERATORS_NP[kind](n, seed)
+
+
+def abs_eb(orc, x, mode, val):
+    if mode == "abs":
+        return np.float32(val)
+    mn, mx = orc.value_range(x)
+    return orc.rel_to_abs(val, mn, mx)
+
+
+def assert_stream_equal(got, want, what):
+    assert got.size == want.size and np.array_equal(got, want), f"{what}: {first_diff(got, want)}"
+
+
+CASES = [
+    ("smooth", 1 << 20, "rel", 1e-4),
+    ("smooth", 1 << 20, "rel", 1e-2),
+    ("smooth", 1 << 18, "rel", 1e-6),
+    ("smooth", 1 << 15, "rel", 1e-3),
+    ("gradient_like", 1 << 20, "abs", 1e-6),
+    ("gradient_like", 1 << 19, "rel", 1e-2),
+    ("gradient_like", 1 << 19, "rel", 1e-4),
+    ("uniform", 1 << 19, "rel", 1e-2),
+    ("uniform", 1 << 19, "rel", 1e-4),
+    ("uniform", 1 << 18, "rel", 1e-6),
+    ("smooth", (1 << 18) + 4096 * 3, "rel", 1e-4),     # whole tiles, ragged chunk
+    ("smooth", (1 << 17) + 8 * 37, "rel", 1e-4),       # ragged tile
+    ("uniform", (1 << 16) + 13, "rel", 1e-4),          # ragged lane group
+    ("gradient_like", 100, "abs", 1e-6),
+    ("uniform", 1, "abs", 1e-3),
+    ("uniform", 31, "abs", 1e-3),
+    ("uniform", 33, "abs", 1e-3),
+    ("smooth", 32768 + 1, "rel", 1e-4),
+]
+
+
+@pytest.mark.parametrize("kind,n,mode,val", CASES)
+def test_compress_decompress(gpu, orc, gen, kind, n, mode, val):
+    x = make(gen, kind, n)
+    eb = abs_eb(orc, x, mode, val)
+    want = orc.compress(x, eb)
+    got = gpu.compress(x, eb)
+    assert_stream_equal(got, want, f"compress {kind} n={n} eb={eb}")
+    want_dec = orc.decompress(want, n, eb)
+    got_dec = gpu.decompress(want, n, eb)
+    assert np.array_equal(got_dec.view(np.uint32), want_dec.view(np.uint32)), "decompressed floats differ"
+    err = np.abs(got_dec.astype(np.float64) - x.astype(np.float64))
+    bound = float(eb) + 2.0 ** -21 * np.abs(x.astype(np.float64))
+    assert (err <= bound).all(), f"error bound violated: {(err / float(eb)).max()} eb"
+
+
+@pytest.mark.parametrize("kind,n,mode,val", CASES[:12])
+def test_hom_sums(gpu, orc, gen, kind, n, mode, val):
+    a = make(gen, kind, n, seed=1)
+    b = make(gen, kind, n, seed=2)
+    eb = abs_eb(orc, np.concatenate([a, b]), mode, val)
+    sa = orc.compress(a, eb)
+    want = orc.hom_sum_f32(sa, b, eb)
+    got = gpu.hom_sum_f32(sa, b, eb)
+    assert_stream_equal(got, want, "hom_sum_f32")
+    # integer homomorphism: decoded quantised values are exactly q(a) + q(b)
+    q = orc.decode_quants(got, n)
+    assert np.array_equal(q, orc.quantize_array(a, eb) + orc.quantize_array(b, eb))
+    # the 2-kernel variant (Lorenzo pre-pass + integer sum) gives the same stream
+    d_gpu = gpu.quant_predict(b, eb)
+    assert np.array_equal(d_gpu, orc.quant_predict(b, eb)), "quant_predict differs"
+    got_i = gpu.hom_sum_i32(sa, d_gpu)
+    assert_stream_equal(got_i, want, "hom_sum_i32")
+    # stream (+) stream
+    sb = orc.compress(b, eb)
+    got_add = gpu.hom_add(sa, sb, n)
+    assert_stream_equal(got_add, orc.hom_add(sa, sb, n), "hom_add vs oracle")
+    assert_stream_equal(got_add, want, "hom_add vs hom_sum_f32")
+    # decompress the sum: within 2*eb (+ float slack) of a + b
+    dec = gpu.decompress(got, n, eb)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
+    s = a.astype(np.float64) + b.astype(np.float64)
+    bound = 2 * float(eb) + 2.0 ** -20 * (np.abs(a) + np.abs(b)).astype(np.float64)
+    assert (np.abs(dec.astype(np.float64) - s) <= bound).all()
+
+
+def rand_deltas(rng, nblocks):
+    """Blocks covering every plane count, both modes and every outlier width."""
+    d = np.zeros((nblocks, 32), np.int64)
+    for b in range(nblocks):
+        F = int(rng.integers(0, 32))
+        mode = int(rng.integers(0, 5))
+        if F:
+            d[b] = rng.integers(0, 1 << F, 32)
+            d[b, rng.integers(1, 32)] |= 1 << (F - 1)
+        if mode == 1:                       # big first element -> outlier mode
+            d[b, 0] = int(rng.integers(1, 1 << int(rng.integers(1, 32))))
+        elif mode == 2:                     # only the first element is non-zero (F = 0 corner)
+            d[b, 1:] = 0
+            d[b, 0] = int(rng.integers(1, 1 << int(rng.integers(1, 32))))
+        elif mode == 3:
+            d[b] = 0
+        sign = rng.integers(0, 2, 32) * 2 - 1
+        d[b] *= sign
+    return d.reshape(-1).astype(np.int32)
+
+
+def test_every_rate_and_mode(gpu, orc):
+    """Crafted deltas through hom_sum_i32 on an all-zero stream: exercises plane counts 0..31,
+    plain and outlier mode, outlier widths 1..4 and negative first elements."""
+    rng = np.random.default_rng(7)
+    n = 1 << 16
+    d = rand_deltas(rng, n // 32)
+    zero = orc.compress(np.zeros(n, np.float32), 1.0)
+    assert zero.size == orc.header_bytes(n)
+    want = orc.encode_deltas(d)
+    got = gpu.hom_sum_i32(zero, d)
+    assert_stream_equal(got, want, "encode of crafted deltas")
+    hdr = got[:orc.header_bytes(n)]
+    assert set(np.unique(hdr & 31)) == set(range(32))
+    assert set(np.unique(hdr[hdr >= 128] >> 5 & 3)) == {0, 1, 2, 3}
+    # decode side: stream (+) stream with the same crafted stream doubles every delta
+    d2 = rand_deltas(np.random.default_rng(8), n // 32) >> 1
+    s2 = orc.encode_deltas(d2)
+    s1 = orc.encode_deltas(d >> 1)
+    got_add = gpu.hom_add(s1, s2, n)
+    assert_stream_equal(got_add, orc.encode_deltas((d >> 1) + d2), "hom_add of crafted streams")
+    # and decompress of the crafted stream (quantised values = running sums)
+    dec = gpu.decompress(s1, n, 0.5)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(s1, n, 0.5).view(np.uint32))
+
+
+def test_zero_incoming_blocks(gpu, orc, gen):
+    """Incoming blocks with a zero header contribute nothing (the reference leaves stale
+    registers there, HomComp/src/homcomp.cu:3086,3149); the local data must still be added."""
+    n = 1 << 17
+    a = gen.gradient_like_np(n, 1)
+    b = gen.smooth_np(n, 2)
+    eb = np.float32(5e-2)                     # coarse: most blocks of `a` quantise to zero
+    sa = orc.compress(a, eb)
+    assert (sa[:orc.header_bytes(n)] == 0).mean() > 0.5
+    got = gpu.hom_sum_f32(sa, b, eb)
+    assert_stream_equal(got, orc.hom_sum_f32(sa, b, eb), "hom_sum_f32 with zero blocks")
+    assert np.array_equal(orc.decode_quants(got, n),
+                          orc.quantize_array(a, eb) + orc.quantize_array(b, eb))
+
+
+@pytest.mark.parametrize("special", ["zeros", "constant", "nan_inf", "huge", "alternating"])
+def test_special_values(gpu, orc, special):
+    n = 1 << 15
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(n).astype(np.float32)
+    eb = np.float32(1e-3)
+    if special == "zeros":
+        x[:] = 0
+    elif special == "constant":
+        x[:] = -3.25
+    elif special == "nan_inf":                 # outside the codec's domain: must stay well defined
+        x[5] = np.nan
+        x[77] = np.inf
+        x[1000] = -np.inf
+    elif special == "huge":
+        x *= 1e6
+        x[::97] = 3e9
+    elif special == "alternating":
+        x = (np.arange(n) % 2 * 2 - 1).astype(np.float32) * 1e4
+    want = orc.compress(x, eb)
+    got = gpu.compress(x, eb)
+    assert_stream_equal(got, want, special)
+    dec = gpu.decompress(want, n, eb)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
+
+
+def test_empty(gpu, pkg, cuda):
+    cmp = gpu.stream_buf(0)
+    dlen = cuda.full((1,), 99, dtype=cuda.int64, device="cuda")
+    x = cuda.zeros(4, dtype=cuda.float32, device="cuda")
+    gpu.ws.compress(x, 1e-3, cmp, stream_len=dlen, n=0)
+    assert gpu.ws.last_size() == 0 and int(dlen.item()) == 0
+    gpu.ws.decompress(cmp, 0, 0, 1e-3, x)
+    cuda.cuda.synchronize()
+
+
+def test_truncated_stream_size(gpu, orc, gen):
+    """Out-of-bound rule (HomComp/src/GSZ.cu:908-911): blocks whose payload starts at or past
+    the stated size are skipped; with the full buffer still in place the rest decodes."""
+    n = 1 << 17
+    x = gen.smooth_np(n, 5)
+    eb = np.float32(1e-3)
+    s = orc.compress(x, eb)
+    for cut in (s.size - 1, s.size - 4097, orc.header_bytes(n) + 10, orc.header_bytes(n)):
+        got = gpu.decompress(s, n, eb, cmp_size=cut)
+        want = orc.decompress(s, n, eb, cmp_size=cut)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"cut={cut}"
+        y = gen.smooth_np(n, 6)
+        got_h = gpu.hom_sum_f32(s, y, eb, cmp_size=cut)
+        assert_stream_equal(got_h, orc.hom_sum_f32(s, y, eb, cmp_in_size=cut), f"hom cut={cut}")
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3, 5, 8, 15])
+def test_unaligned_stream_pointers(gpu, orc, gen, offset):
+    n = 1 << 16
+    x = gen.smooth_np(n, 9)
+    y = gen.uniform_np(n, 10)
+    eb = np.float32(2e-4)
+    want = orc.compress(x, eb)
+    assert_stream_equal(gpu.compress(x, eb, offset=offset), want, "compress")
+    dec = gpu.decompress(want, n, eb, offset=offset)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
+    assert_stream_equal(gpu.hom_sum_f32(want, y, eb, offset=offset), orc.hom_sum_f32(want, y, eb), "hom")
+
+
+def test_value_range(gpu, orc, gen, pkg):
+    for kind, n in (("smooth", 1 << 20), ("uniform", 12345), ("gradient_like", 7)):
+        x = make(gen, kind, n, seed=4)
+        mn, mx = gpu.value_range(x)
+        omn, omx = orc.value_range(x)
+        assert mn == omn == x.min() and mx == omx == x.max()
+        assert np.float32(pkg.rel_to_abs(1e-4, mn, mx)) == orc.rel_to_abs(1e-4, mn, mx)
+
+
+def test_workspace_reuse_many_calls(gpu, orc, gen):
+    """The status words are never cleared between calls; sizes shrink and grow to make stale
+    words of earlier calls visible to later ones."""
+    eb = np.float32(1e-3)
+    for i, n in enumerate([1 << 20, 1 << 15, 1 << 18, 4096, 1 << 20, 1 << 16]):
+        x = gen.uniform_np(n, 20 + i)
+        assert_stream_equal(gpu.compress(x, eb), orc.compress(x, eb), f"call {i}")
+
+
+def test_argument_errors(gpu, pkg, cuda):
+    x = cuda.zeros(64, dtype=cuda.float32, device="cuda")
+    cmp = gpu.stream_buf(64)
+    L = pkg.lib()
+    import ctypes as C
+    h = gpu.ws._h
+    assert L.homcomp_compress_f32(h, x.data_ptr(), 64, C.c_float(0.0), cmp.data_ptr(), None, None) == -1
+    assert L.homcomp_compress_f32(h, x.data_ptr(), 64, C.c_float(float("nan")), cmp.data_ptr(), None, None) == -1
+    assert L.homcomp_compress_f32(h, x.data_ptr() + 4, 32, C.c_float(1e-3), cmp.data_ptr(), None, None) == -2
+    assert L.homcomp_compress_f32(h, x.data_ptr(), MAX_N + 1, C.c_float(1e-3), cmp.data_ptr(), None, None) == -3
+    assert L.homcomp_compress_f32(None, x.data_ptr(), 64, C.c_float(1e-3), cmp.data_ptr(), None, None) == -1
+    assert L.homcomp_compress_f32(h, None, 64, C.c_float(1e-3), cmp.data_ptr(), None, None) == -1
+    assert pkg.status_string(-2).startswith("float")

@@ -1,0 +1,179 @@
+"""MI355X-native HomComp: ctypes binding of libhomcomp_amd.so (the C ABI of include/homcomp.h).
+
+The directory name is not a valid Python identifier; load it with ``__graft_entry__.load_package()``
+(it registers the module as ``tirocinio_triennale_amd``).
+
+There is no CPU fallback: if the HIP library is missing or no GPU is present every call raises.
+torch is used for device memory and streams only; all codec work happens in the HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhomcomp_amd.so")
+
+# every symbol include/homcomp.h declares
+EXPORTS = (
+    "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
+    "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
+    "homcomp_workspace_destroy", "homcomp_compress_f32", "homcomp_decompress_f32",
+    "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add",
+    "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
+)
+
+
+class HomCompError(RuntimeError):
+    def __init__(self, status: int, what: str):
+        self.status = status
+        super().__init__(f"{what}: {status_string(status)} (status {status}, "
+                         f"hip error {lib().homcomp_last_hip_error()})")
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Load the HIP library; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                f"(python tirocinio-triennale_amd/build.py)")
+        L = C.CDLL(LIB_PATH)
+        vp, sz, u64p = C.c_void_p, C.c_size_t, C.c_void_p
+        L.homcomp_status_string.argtypes = [C.c_int]
+        L.homcomp_status_string.restype = C.c_char_p
+        L.homcomp_last_hip_error.restype = C.c_int
+        for name in ("homcomp_header_bytes", "homcomp_max_stream_bytes"):
+            getattr(L, name).argtypes = [sz]
+            getattr(L, name).restype = sz
+        L.homcomp_ref_cmpsize.argtypes = [sz, sz]
+        L.homcomp_ref_cmpsize.restype = sz
+        L.homcomp_workspace_create.argtypes = [C.POINTER(vp), sz]
+        L.homcomp_workspace_destroy.argtypes = [vp]
+        L.homcomp_compress_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
+        L.homcomp_decompress_f32.argtypes = [vp, vp, sz, sz, C.c_float, vp, vp]
+        L.homcomp_hom_sum_f32.argtypes = [vp, vp, sz, vp, sz, C.c_float, vp, u64p, vp]
+        L.homcomp_hom_sum_i32.argtypes = [vp, vp, sz, vp, sz, vp, u64p, vp]
+        L.homcomp_hom_add.argtypes = [vp, vp, sz, vp, sz, sz, vp, u64p, vp]
+        L.homcomp_quant_predict_f32.argtypes = [vp, sz, C.c_float, vp, vp]
+        L.homcomp_range_f32.argtypes = [vp, vp, sz, vp, vp]
+        L.homcomp_rel_to_abs.argtypes = [C.c_float, C.c_float, C.c_float]
+        L.homcomp_rel_to_abs.restype = C.c_float
+        L.homcomp_last_size.argtypes = [vp, C.POINTER(sz), vp]
+        _lib = L
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return lib().homcomp_status_string(status).decode()
+
+
+def header_bytes(n: int) -> int:
+    return int(lib().homcomp_header_bytes(n))
+
+
+def max_stream_bytes(n: int) -> int:
+    return int(lib().homcomp_max_stream_bytes(n))
+
+
+def ref_cmpsize(stream_len: int, n: int) -> int:
+    return int(lib().homcomp_ref_cmpsize(stream_len, n))
+
+
+def rel_to_abs(rel: float, vmin: float, vmax: float) -> float:
+    return float(lib().homcomp_rel_to_abs(rel, vmin, vmax))
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise HomCompError(status, what)
+
+
+def _stream_ptr(stream) -> int:
+    import torch
+    s = torch.cuda.current_stream() if stream is None else stream
+    return int(s.cuda_stream)
+
+
+class Workspace:
+    """Scan state for one in-flight call (homcomp_workspace_create / _destroy).
+
+    Methods take torch CUDA tensors, enqueue on ``stream`` (default: torch's current stream)
+    and return immediately; ``last_size`` is the only blocking call.
+    """
+
+    def __init__(self, max_n: int):
+        self._h = C.c_void_p()
+        self.max_n = int(max_n)
+        _check(lib().homcomp_workspace_create(C.byref(self._h), self.max_n), "workspace_create")
+
+    def close(self) -> None:
+        if self._h:
+            _check(lib().homcomp_workspace_destroy(self._h), "workspace_destroy")
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- raw entry points (tensor arguments, explicit sizes) ---------------------------------
+    def compress(self, data, eb: float, cmp, stream_len=None, n: int | None = None, stream=None):
+        n = data.numel() if n is None else n
+        _check(lib().homcomp_compress_f32(self._h, data.data_ptr(), n, eb, cmp.data_ptr(),
+                                          stream_len.data_ptr() if stream_len is not None else None,
+                                          _stream_ptr(stream)), "compress_f32")
+
+    def decompress(self, cmp, cmp_size: int, n: int, eb: float, out, stream=None):
+        _check(lib().homcomp_decompress_f32(self._h, cmp.data_ptr(), cmp_size, n, eb,
+                                            out.data_ptr(), _stream_ptr(stream)), "decompress_f32")
+
+    def hom_sum_f32(self, cmp_in, cmp_in_size: int, local, eb: float, cmp_out, stream_len=None,
+                    n: int | None = None, stream=None):
+        n = local.numel() if n is None else n
+        _check(lib().homcomp_hom_sum_f32(self._h, cmp_in.data_ptr(), cmp_in_size, local.data_ptr(),
+                                         n, eb, cmp_out.data_ptr(),
+                                         stream_len.data_ptr() if stream_len is not None else None,
+                                         _stream_ptr(stream)), "hom_sum_f32")
+
+    def hom_sum_i32(self, cmp_in, cmp_in_size: int, local_delta, cmp_out, stream_len=None,
+                    n: int | None = None, stream=None):
+        n = local_delta.numel() if n is None else n
+        _check(lib().homcomp_hom_sum_i32(self._h, cmp_in.data_ptr(), cmp_in_size,
+                                         local_delta.data_ptr(), n, cmp_out.data_ptr(),
+                                         stream_len.data_ptr() if stream_len is not None else None,
+                                         _stream_ptr(stream)), "hom_sum_i32")
+
+    def hom_add(self, cmp_a, size_a: int, cmp_b, size_b: int, n: int, cmp_out, stream_len=None,
+                stream=None):
+        _check(lib().homcomp_hom_add(self._h, cmp_a.data_ptr(), size_a, cmp_b.data_ptr(), size_b,
+                                     n, cmp_out.data_ptr(),
+                                     stream_len.data_ptr() if stream_len is not None else None,
+                                     _stream_ptr(stream)), "hom_add")
+
+    def value_range(self, data, minmax, n: int | None = None, stream=None):
+        n = data.numel() if n is None else n
+        _check(lib().homcomp_range_f32(self._h, data.data_ptr(), n, minmax.data_ptr(),
+                                       _stream_ptr(stream)), "range_f32")
+
+    def last_size(self, stream=None) -> int:
+        out = C.c_size_t()
+        _check(lib().homcomp_last_size(self._h, C.byref(out), _stream_ptr(stream)), "last_size")
+        return int(out.value)
+
+
+def quant_predict(data, eb: float, delta, n: int | None = None, stream=None) -> None:
+    n = data.numel() if n is None else n
+    _check(lib().homcomp_quant_predict_f32(data.data_ptr(), n, eb, delta.data_ptr(),
+                                           _stream_ptr(stream)), "quant_predict_f32")

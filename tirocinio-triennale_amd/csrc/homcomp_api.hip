@@ -1,0 +1,317 @@
+// C ABI of libhomcomp_amd.so: argument checking, workspace management and launch geometry.
+// The interface is documented in include/homcomp.h.
+#include "../../include/homcomp.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+#include <new>
+
+#include "homcomp_kernels.hpp"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+constexpr uint32_t kMaxEpoch = (1u << 22) - 1;
+constexpr uint32_t kRangePartials = 2048;
+
+inline bool hip_ok(hipError_t e)
+{
+    if (e == hipSuccess) return true;
+    g_last_hip_error = (int)e;
+    return false;
+}
+
+inline size_t chunks_of(size_t n) { return (n + hc::kHostChunkElems - 1) / hc::kHostChunkElems; }
+inline size_t padded_len(size_t n) { return chunks_of(n) * hc::kHostChunkElems; }
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+inline bool eb_ok(float eb) { return std::isfinite(eb) && eb > 0.0f; }
+
+}  // namespace
+
+struct homcomp_workspace {
+    int device;
+    size_t max_n;
+    uint32_t max_tiles;
+    void *d_block;          // one allocation: status[3][max_tiles] | total | ticket | range partials
+    uint64_t *d_status[3];
+    uint64_t *d_total;
+    uint32_t *d_ticket;
+    float *d_partial;
+    uint64_t *h_total;      // pinned host word for the blocking size read-back
+    uint32_t epoch;         // last epoch handed out (1..kMaxEpoch)
+    uint32_t ticket_base;   // value of *d_ticket once all enqueued launches have run
+};
+
+namespace {
+
+int check_ws(const homcomp_workspace *ws, size_t n)
+{
+    if (!ws) return HOMCOMP_ERR_INVALID_ARG;
+    if (n > ws->max_n) return HOMCOMP_ERR_TOO_LARGE;
+    int dev = -1;
+    if (!hip_ok(hipGetDevice(&dev))) return HOMCOMP_ERR_HIP;
+    if (dev != ws->device) return HOMCOMP_ERR_INVALID_ARG;
+    return HOMCOMP_OK;
+}
+
+// Fresh epoch for one launch; clears the status words when the 22-bit tag wraps.
+int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
+{
+    if (ws->epoch >= kMaxEpoch) {
+        if (!hip_ok(hc::launch_fill_u64(ws->d_status[0], (uint64_t)ws->max_tiles * 3, s)))
+            return HOMCOMP_ERR_HIP;
+        ws->epoch = 0;
+    }
+    *epoch = ++ws->epoch;
+    return HOMCOMP_OK;
+}
+
+int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *p)
+{
+    std::memset(p, 0, sizeof *p);
+    p->n = n;
+    p->hdr_bytes = homcomp_header_bytes(n);
+    p->n_tiles = (uint32_t)(padded_len(n) / hc::kHostTileElems);
+    for (int c = 0; c < 3; ++c) p->status[c] = ws->d_status[c];
+    p->ticket = ws->d_ticket;
+    p->ticket_base = ws->ticket_base;
+    ws->ticket_base += p->n_tiles;
+    p->total = ws->d_total;
+    return next_epoch(ws, s, &p->epoch);
+}
+
+// n == 0: the stream is empty; only the length words are written.
+int empty_stream(homcomp_workspace *ws, uint64_t *d_stream_len, hipStream_t s)
+{
+    if (!hip_ok(hc::launch_fill_u64(ws->d_total, 1, s))) return HOMCOMP_ERR_HIP;
+    if (d_stream_len && !hip_ok(hc::launch_fill_u64(d_stream_len, 1, s))) return HOMCOMP_ERR_HIP;
+    return HOMCOMP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *homcomp_status_string(int status)
+{
+    switch (status) {
+    case HOMCOMP_OK: return "ok";
+    case HOMCOMP_ERR_INVALID_ARG: return "invalid argument";
+    case HOMCOMP_ERR_ALIGNMENT: return "float/int32 buffer not 16-byte aligned";
+    case HOMCOMP_ERR_TOO_LARGE: return "nbEle exceeds the workspace capacity";
+    case HOMCOMP_ERR_HIP: return "HIP runtime error";
+    case HOMCOMP_ERR_NO_DEVICE: return "no usable GPU";
+    default: return "unknown status";
+    }
+}
+
+int homcomp_last_hip_error(void) { return g_last_hip_error; }
+
+size_t homcomp_header_bytes(size_t nbEle) { return chunks_of(nbEle) * (hc::kHostChunkElems / 32); }
+
+size_t homcomp_max_stream_bytes(size_t nbEle)
+{
+    const size_t blocks = homcomp_header_bytes(nbEle);
+    return blocks + blocks * 128u;
+}
+
+size_t homcomp_ref_cmpsize(size_t stream_len, size_t nbEle) { return stream_len + homcomp_header_bytes(nbEle); }
+
+float homcomp_rel_to_abs(float rel, float vmin, float vmax)
+{
+    volatile float range = vmax - vmin;
+    volatile float eb = rel * range;
+    return eb;
+}
+
+int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
+{
+    if (!out) return HOMCOMP_ERR_INVALID_ARG;
+    *out = nullptr;
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) {
+        (void)hipGetLastError();
+        return HOMCOMP_ERR_NO_DEVICE;
+    }
+    const size_t tiles = padded_len(max_nbEle) / hc::kHostTileElems;
+    if (tiles >= (1ull << 31)) return HOMCOMP_ERR_TOO_LARGE;
+    homcomp_workspace *ws = new (std::nothrow) homcomp_workspace();
+    if (!ws) return HOMCOMP_ERR_INVALID_ARG;
+    std::memset(ws, 0, sizeof *ws);
+    ws->max_n = max_nbEle;
+    ws->max_tiles = (uint32_t)(tiles ? tiles : 1);
+    if (!hip_ok(hipGetDevice(&ws->device))) {
+        delete ws;
+        return HOMCOMP_ERR_HIP;
+    }
+    const size_t status_bytes = (size_t)ws->max_tiles * 3 * sizeof(uint64_t);
+    const size_t bytes = status_bytes + 256 + kRangePartials * 2 * sizeof(float);
+    if (!hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
+        !hip_ok(hipHostMalloc((void **)&ws->h_total, sizeof(uint64_t), hipHostMallocDefault))) {
+        if (ws->d_block) (void)hipFree(ws->d_block);
+        delete ws;
+        return HOMCOMP_ERR_HIP;
+    }
+    uint8_t *base = (uint8_t *)ws->d_block;
+    for (int c = 0; c < 3; ++c) ws->d_status[c] = (uint64_t *)base + (size_t)c * ws->max_tiles;
+    ws->d_total = (uint64_t *)(base + status_bytes);
+    ws->d_ticket = (uint32_t *)(base + status_bytes + 128);
+    ws->d_partial = (float *)(base + status_bytes + 256);
+    *out = ws;
+    return HOMCOMP_OK;
+}
+
+int homcomp_workspace_destroy(homcomp_workspace *ws)
+{
+    if (!ws) return HOMCOMP_OK;
+    int rc = HOMCOMP_OK;
+    if (!hip_ok(hipDeviceSynchronize())) rc = HOMCOMP_ERR_HIP;
+    if (!hip_ok(hipFree(ws->d_block))) rc = HOMCOMP_ERR_HIP;
+    if (!hip_ok(hipHostFree(ws->h_total))) rc = HOMCOMP_ERR_HIP;
+    delete ws;
+    return rc;
+}
+
+int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float eb,
+                         unsigned char *d_cmp, uint64_t *d_stream_len, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
+    if (!d_data || !d_cmp) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_data)) return HOMCOMP_ERR_ALIGNMENT;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.local = d_data;
+    p.out_cmp = d_cmp;
+    p.eb = eb;
+    p.recip = 0.5f / eb;
+    p.user_total = d_stream_len;
+    return hip_ok(hc::launch_compress(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
+                           size_t nbEle, float eb, float *d_out, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle == 0) return HOMCOMP_OK;
+    if (!d_cmp || !d_out) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_out)) return HOMCOMP_ERR_ALIGNMENT;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.in[0] = d_cmp;
+    p.in_size[0] = cmp_size;
+    p.out_f32 = d_out;
+    p.eb = eb;
+    p.recip = 0.5f / eb;
+    return hip_ok(hc::launch_decompress(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
+                        const float *d_local, size_t nbEle, float eb, unsigned char *d_cmp_out,
+                        uint64_t *d_stream_len, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
+    if (!d_cmp_in || !d_local || !d_cmp_out) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_local)) return HOMCOMP_ERR_ALIGNMENT;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.in[0] = d_cmp_in;
+    p.in_size[0] = cmp_in_size;
+    p.local = d_local;
+    p.out_cmp = d_cmp_out;
+    p.eb = eb;
+    p.recip = 0.5f / eb;
+    p.user_total = d_stream_len;
+    return hip_ok(hc::launch_hom_sum_f32(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
+                        const int32_t *d_local_delta, size_t nbEle, unsigned char *d_cmp_out,
+                        uint64_t *d_stream_len, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
+    if (!d_cmp_in || !d_local_delta || !d_cmp_out) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_local_delta)) return HOMCOMP_ERR_ALIGNMENT;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.in[0] = d_cmp_in;
+    p.in_size[0] = cmp_in_size;
+    p.local = d_local_delta;
+    p.out_cmp = d_cmp_out;
+    p.user_total = d_stream_len;
+    return hip_ok(hc::launch_hom_sum_i32(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t size_a,
+                    const unsigned char *d_cmp_b, size_t size_b, size_t nbEle,
+                    unsigned char *d_cmp_out, uint64_t *d_stream_len, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
+    if (!d_cmp_a || !d_cmp_b || !d_cmp_out) return HOMCOMP_ERR_INVALID_ARG;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.in[0] = d_cmp_a;
+    p.in_size[0] = size_a;
+    p.in[1] = d_cmp_b;
+    p.in_size[1] = size_b;
+    p.out_cmp = d_cmp_out;
+    p.user_total = d_stream_len;
+    return hip_ok(hc::launch_hom_add(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,
+                              void *stream)
+{
+    if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle == 0) return HOMCOMP_OK;
+    if (!d_data || !d_delta) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_data) || !aligned16(d_delta)) return HOMCOMP_ERR_ALIGNMENT;
+    return hip_ok(hc::launch_quant_predict(d_data, d_delta, nbEle, 0.5f / eb, (hipStream_t)stream))
+               ? HOMCOMP_OK
+               : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_range_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float *d_minmax,
+                      void *stream)
+{
+    int rc = check_ws(ws, 0);
+    if (rc) return rc;
+    if (!d_data || !d_minmax || nbEle == 0) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_data)) return HOMCOMP_ERR_ALIGNMENT;
+    return hip_ok(hc::launch_range(d_data, nbEle, ws->d_partial, kRangePartials, d_minmax,
+                                   (hipStream_t)stream))
+               ? HOMCOMP_OK
+               : HOMCOMP_ERR_HIP;
+}
+
+int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream)
+{
+    if (!ws || !stream_len) return HOMCOMP_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (!hip_ok(hipMemcpyAsync(ws->h_total, ws->d_total, sizeof(uint64_t), hipMemcpyDeviceToHost, s)) ||
+        !hip_ok(hipStreamSynchronize(s)))
+        return HOMCOMP_ERR_HIP;
+    *stream_len = (size_t)*ws->h_total;
+    return HOMCOMP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,309 @@
+// Device-side building blocks of the HomComp codec for gfx950 (wave64).
+//
+// Work mapping (differs on purpose from the reference's one-thread-per-block, 32-thread layout,
+// HomComp/include/GSZ.h:4-9): a 32-element block is owned by 4 adjacent lanes, 8 consecutive
+// elements per lane.  One lane therefore produces exactly one byte of every bit plane (the
+// stream stores plane p as 4 bytes, byte k covering elements 8k..8k+7 MSB first,
+// HomComp/src/GSZ.cu:312-351), and an 8x8 bit-matrix transpose turns its eight magnitudes
+// into eight plane bytes at once.  Cross-lane traffic is limited to quad-local DPP moves.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hc {
+
+constexpr int kWG = 256;                              // threads per workgroup (4 waves)
+constexpr int kEPL = 8;                               // elements per lane per iteration
+constexpr int kQuad = 4;                              // lanes per 32-element block
+constexpr int kIter = 2;                              // iterations per tile
+constexpr int kBlocksPerIter = kWG / kQuad;           // 64
+constexpr int kTileBlocks = kBlocksPerIter * kIter;   // 128
+constexpr int kTileElems = kTileBlocks * 32;          // 4096
+constexpr int kChunkElems = 32768;                    // reference thread-block share
+constexpr int kMaxBlockBytes = 132;                   // largest size a header byte can imply
+constexpr int kStageBytes = kTileBlocks * kMaxBlockBytes + 64;
+
+// ---------------------------------------------------------------- cross-lane helpers
+
+// Quad-local lane permutation through DPP; must run with all lanes of the wave active.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+constexpr int kDppXor1 = 0xB1;      // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;      // quad_perm [2,3,0,1]
+constexpr int kDppBcast0 = 0x00;    // quad_perm [0,0,0,0]
+constexpr int kDppBcast1 = 0x55;    // quad_perm [1,1,1,1]
+constexpr int kDppBcast2 = 0xAA;    // quad_perm [2,2,2,2]
+constexpr int kDppRowShr1 = 0x111;  // lane i reads lane i-1 inside its row of 16 (0 at row start)
+
+__device__ __forceinline__ uint32_t quad_or(uint32_t v)
+{
+    v |= dpp_u32<kDppXor1>(v);
+    v |= dpp_u32<kDppXor2>(v);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int lane)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        uint32_t t = __shfl_up(x, d, 64);
+        if (lane >= d) x += t;
+    }
+    return x;
+}
+
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t x)
+{
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        uint32_t lo = __shfl_xor((uint32_t)x, d, 64);
+        uint32_t hi = __shfl_xor((uint32_t)(x >> 32), d, 64);
+        x += ((uint64_t)hi << 32) | lo;
+    }
+    return x;
+}
+
+// ---------------------------------------------------------------- scalar arithmetic
+
+// HomComp/src/GSZ.cu:6-25: fl(x*r), compare with -0.5, fl(.+0.5), convert toward zero
+// (saturating, NaN -> 0, which v_cvt_i32_f32 does as PTX cvt.rzi.s32.f32 does), wrapping subtract.
+__device__ __forceinline__ int32_t quantize(float x, float recip)
+{
+    float d = __fmul_rn(x, recip);
+    uint32_t s = (d >= -0.5f) ? 0u : 1u;
+    float t = __fadd_rn(d, 0.5f);
+    int32_t r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(t));
+    return (int32_t)((uint32_t)r - s);
+}
+
+// HomComp/src/GSZ.cu:1437: currQuant * eb * 2, two float32 multiplications.
+__device__ __forceinline__ float dequantize(int32_t q, float eb)
+{
+    return __fmul_rn(__fmul_rn((float)q, eb), 2.0f);
+}
+
+// HomComp/src/GSZ.cu:27-31
+__device__ __forceinline__ uint32_t bit_num(uint32_t x) { return 32u - (uint32_t)__clz((int)x); }
+
+// Plane count of a block maximum; the 5-bit header field caps it at 31.
+__device__ __forceinline__ uint32_t planes_of(uint32_t m)
+{
+    uint32_t b = bit_num(m);
+    return b > 31u ? 31u : b;
+}
+
+// HomComp/src/GSZ.cu:795-802: payload bytes implied by a header byte.
+__device__ __forceinline__ uint32_t size_from_header(uint32_t h)
+{
+    uint32_t F = h & 0x1fu;
+    uint32_t ob = ((h >> 5) & 3u) + 1u;
+    return (h & 0x80u) ? 4u + 4u * F + ob : (F ? 4u + 4u * F : 0u);
+}
+
+// Transpose of an 8x8 bit matrix held row-per-byte: result bit (8r+c) = input bit (8c+r).
+__device__ __forceinline__ uint64_t transpose8(uint64_t x)
+{
+    uint64_t t;
+    t = (x ^ (x >> 7)) & 0x00AA00AA00AA00AAull;
+    x = x ^ t ^ (t << 7);
+    t = (x ^ (x >> 14)) & 0x0000CCCC0000CCCCull;
+    x = x ^ t ^ (t << 14);
+    t = (x ^ (x >> 28)) & 0x00000000F0F0F0F0ull;
+    x = x ^ t ^ (t << 28);
+    return x;
+}
+
+// ---------------------------------------------------------------- per-lane block pieces
+
+// Encoder front end for one lane's 8 signed deltas (HomComp/src/GSZ.cu:86-164): sign byte,
+// magnitudes, block-wide bit widths through the quad, rate selection.  `k` is the lane's
+// position in its quad.  hdr and size come out identical in the four lanes of a quad.
+__device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8], uint32_t &sb,
+                                         uint32_t &hdr, uint32_t &size)
+{
+    sb = 0;
+    uint32_t rest = 0;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        uint32_t neg = v[m] < 0 ? 1u : 0u;
+        a[m] = neg ? 0u - (uint32_t)v[m] : (uint32_t)v[m];
+        sb |= neg << (7 - m);
+        if (m) rest |= a[m];
+    }
+    // bit width of a maximum equals the bit width of the OR
+    uint32_t or1 = quad_or(rest | a[0]);                  // all 32 elements   (:152)
+    uint32_t or2 = quad_or(rest | (k ? a[0] : 0u));       // elements 1..31    (:153)
+    uint32_t a0 = dpp_u32<kDppBcast0>(a[0]);              // element 0         (:154)
+    uint32_t fr1 = planes_of(or1);
+    uint32_t fr2 = planes_of(or2);
+    uint32_t ob = (bit_num(a0) + 7u) >> 3;
+    uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;              // :156
+    uint32_t sz2 = 4u + 4u * fr2 + ob;                    // :157
+    if (sz1 <= sz2) {                                     // :158-160
+        hdr = fr1;
+        size = sz1;
+    } else {                                              // :161-164
+        hdr = fr2 | 0x80u | ((ob - 1u) << 5);
+        size = sz2;
+    }
+}
+
+// Encoder back end for one lane (HomComp/src/GSZ.cu:245-751): writes this lane's share of the
+// block payload into the LDS stage at `pos0` (the block's tile-relative offset).  Lane k
+// contributes byte k of the sign word and of every plane; lane 0 also writes the outlier bytes.
+__device__ __forceinline__ void pack8(uint8_t *stage, uint32_t pos0, uint32_t hdr, int k,
+                                      uint32_t a[8], uint32_t sb)
+{
+    const uint32_t sel = hdr >> 7;
+    const uint32_t F = hdr & 0x1fu;
+    if (!sel && F == 0) return;                           // zero block (:287)
+    uint32_t pos = pos0;
+    if (sel) {
+        const uint32_t ob = ((hdr >> 5) & 3u) + 1u;
+        if (k == 0) {
+            uint32_t a0 = a[0];
+            for (uint32_t i = 0; i < ob; ++i) {           // little-endian outlier (:271-275)
+                stage[pos0 + i] = (uint8_t)a0;
+                a0 >>= 8;
+            }
+            a[0] = 0;                                     // element 0 leaves the planes (:274)
+        }
+        pos += ob;
+    }
+    stage[pos + k] = (uint8_t)sb;                         // sign word, MSB = element 0 (:292-295)
+    pos += 4 + k;
+    const uint32_t groups = (F + 7u) >> 3;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        if ((uint32_t)g < groups) {
+            // byte r of x = bits 8g..8g+7 of a[7-r]; after the transpose byte r is plane 8g+r
+            uint32_t lo = ((a[7] >> (8 * g)) & 0xffu) | (((a[6] >> (8 * g)) & 0xffu) << 8) |
+                          (((a[5] >> (8 * g)) & 0xffu) << 16) | (((a[4] >> (8 * g)) & 0xffu) << 24);
+            uint32_t hi = ((a[3] >> (8 * g)) & 0xffu) | (((a[2] >> (8 * g)) & 0xffu) << 8) |
+                          (((a[1] >> (8 * g)) & 0xffu) << 16) | (((a[0] >> (8 * g)) & 0xffu) << 24);
+            uint64_t y = transpose8(((uint64_t)hi << 32) | lo);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                if ((uint32_t)(8 * g + r) < F)
+                    stage[pos + 4u * (uint32_t)(8 * g + r)] = (uint8_t)(y >> (8 * r));
+            }
+        }
+    }
+}
+
+// Decoder for one lane (HomComp/src/GSZ.cu:883-1434 up to the signed deltas): reads this lane's
+// bytes of the block payload at `pos0` in the LDS stage.  Inactive blocks (rate 0, or payload
+// offset beyond the stated stream size, :908-911) give zero deltas.
+__device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uint32_t hdr,
+                                        bool active, int k, int32_t v[8])
+{
+    uint32_t a[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) a[m] = 0;
+    uint32_t sb = 0;
+    if (active) {
+        const uint32_t sel = hdr >> 7;
+        const uint32_t F = hdr & 0x1fu;
+        const uint32_t ob = sel ? ((hdr >> 5) & 3u) + 1u : 0u;
+        uint32_t pos = pos0 + ob;
+        sb = stage[pos + k];                              // :921-924, :990-994
+        pos += 4 + k;
+        const uint32_t groups = (F + 7u) >> 3;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if ((uint32_t)g < groups) {
+                uint64_t y = 0;
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    if ((uint32_t)(8 * g + r) < F)
+                        y |= (uint64_t)stage[pos + 4u * (uint32_t)(8 * g + r)] << (8 * r);
+                }
+                uint64_t x = transpose8(y);
+#pragma unroll
+                for (int r = 0; r < 8; ++r)
+                    a[7 - r] |= (uint32_t)((x >> (8 * r)) & 0xffu) << (8 * g);
+            }
+        }
+        if (sel && k == 0) {                              // :913-917, :986-987, :1005-1006
+            uint32_t o = 0;
+            for (uint32_t i = 0; i < ob; ++i) o |= (uint32_t)stage[pos0 + i] << (8 * i);
+            a[0] = o;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {                         // :1432-1434
+        uint32_t neg = (sb >> (7 - m)) & 1u;
+        v[m] = (int32_t)(neg ? 0u - a[m] : a[m]);
+    }
+}
+
+// ---------------------------------------------------------------- tile status words
+//
+// One 64-bit word per tile and scan chain: bits 63-62 state (0 empty, 1 tile aggregate,
+// 2 inclusive prefix), bits 61-40 the call's epoch, bits 39-0 the byte count.  A word whose
+// epoch is not the current call's reads as empty, so the array never needs clearing between
+// calls (the host clears it when the 22-bit epoch wraps).
+
+constexpr uint64_t kValueMask = (1ull << 40) - 1;
+constexpr uint32_t kEpochMask = (1u << 22) - 1;
+
+__device__ __forceinline__ uint64_t status_word(uint32_t epoch, uint32_t state, uint64_t value)
+{
+    return ((uint64_t)state << 62) | ((uint64_t)(epoch & kEpochMask) << 40) | (value & kValueMask);
+}
+
+__device__ __forceinline__ uint64_t status_load(const uint64_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void status_store(uint64_t *p, uint64_t w)
+{
+    __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Decoupled look-back over the tile status words, run by one full wave.  Publishes this
+// tile's aggregate, sums the aggregates of the predecessors back to the nearest published
+// inclusive prefix (64 predecessors per probe), publishes this tile's inclusive prefix and
+// returns its exclusive prefix.  Tiles take their index from a ticket counter, so every
+// predecessor is already running when a tile starts to wait.
+__device__ __forceinline__ uint64_t lookback(uint64_t *status, uint32_t tile, uint32_t epoch,
+                                             uint64_t aggregate, int lane)
+{
+    if (tile == 0) {
+        if (lane == 0) status_store(&status[0], status_word(epoch, 2, aggregate));
+        return 0;
+    }
+    if (lane == 0) status_store(&status[tile], status_word(epoch, 1, aggregate));
+    uint64_t excl = 0;
+    int64_t base = (int64_t)tile - 1;
+    for (;;) {
+        const int64_t idx = base - lane;
+        uint64_t w = 0;
+        uint32_t st = 2;                                  // virtual zero prefix before tile 0
+        if (idx >= 0) {
+            w = status_load(&status[idx]);
+            st = (((uint32_t)(w >> 40)) & kEpochMask) == (epoch & kEpochMask) ? (uint32_t)(w >> 62) : 0u;
+        }
+        const uint64_t m_empty = __ballot(st == 0);
+        const uint64_t m_prefix = __ballot(st == 2);
+        const int first = m_prefix ? __builtin_ctzll(m_prefix) : 63;
+        const uint64_t need = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
+        if (m_empty & need) {
+            __builtin_amdgcn_s_sleep(2);
+            continue;
+        }
+        excl += wave_sum_u64(lane <= first ? (w & kValueMask) : 0ull);
+        if (m_prefix) break;
+        base -= 64;
+    }
+    if (lane == 0) status_store(&status[tile], status_word(epoch, 2, excl + aggregate));
+    return excl;
+}
+
+}  // namespace hc
