@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the HomComp hot path on one MI355X.
+
+A step is one pass of the hot path over one batch: ``compress`` of a 1 GiB float32 buffer
+followed by ``hom_sum_f32`` of the resulting stream with a second 1 GiB buffer (the compute of
+one ring-allreduce step: a rank compresses its chunk, the next rank adds its own data in the
+quantised domain).  Inputs are resident in HBM before the timed region.  The reported value is
+GB/s of uncompressed input consumed (two 4N-byte operands per step).  Per-operation rates
+(compress, decompress, hom_sum_f32, hom_add) with their roofline fractions are in ``ops``.
+
+Prints one JSON line.  ``--gpus`` above 1 is refused: this build measures one GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X published peak
+
+
+def time_op(torch, fn, iters: int) -> float:
+    """Average kernel-side milliseconds per call, HIP events on the launch stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(orc, x_np, y_np, eb, budget_s: float = 20.0):
+    """The oracle (a C port of the reference's per-block algorithm, OpenMP over 32768-element
+    chunks) on a bounded sample of the same workload, on this host's cores."""
+    import numpy as np
+    threads = min(16, os.cpu_count() or 1)
+    orc.set_threads(threads)
+    n = x_np.size
+    t0 = time.perf_counter()
+    sa = orc.compress(x_np, eb)
+    t1 = time.perf_counter()
+    ss = orc.hom_sum_f32(sa, y_np, eb)
+    t2 = time.perf_counter()
+    best_c, best_h = t1 - t0, t2 - t1
+    reps = 0
+    while time.perf_counter() - t0 < budget_s and reps < 4:
+        a = time.perf_counter()
+        orc.compress(x_np, eb)
+        b = time.perf_counter()
+        orc.hom_sum_f32(sa, y_np, eb)
+        c = time.perf_counter()
+        best_c, best_h = min(best_c, b - a), min(best_h, c - b)
+        reps += 1
+    value = 2 * 4 * n / (best_c + best_h) / 1e9
+    return {
+        "value": round(value, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"first {n} elements of the same workload, compress + hom_sum_f32, best of {reps + 1}",
+        "compress_GBps": round(4 * n / best_c / 1e9, 3),
+        "hom_sum_f32_GBps": round(4 * n / best_h / 1e9, 3),
+    }, sa, ss
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--log2n", type=int, default=28, help="elements per buffer = 2^log2n")
+    ap.add_argument("--kind", default="smooth", choices=["smooth", "gradient_like", "uniform"])
+    ap.add_argument("--rel", type=float, default=1e-4, help="value-range-relative error bound")
+    ap.add_argument("--abs", type=float, default=None, help="absolute error bound (overrides --rel)")
+    ap.add_argument("--cpu-sample-log2", type=int, default=24)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; --gpus above 1 is not part of this build "
+              "(the sharding is described in DESIGN.md)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    pkg = entry.load_package()
+    gen = entry.load_datagen()
+    torch.cuda.set_device(0)
+    n = 1 << args.log2n
+    x = gen.GENERATORS_TORCH[args.kind](n, seed=1)
+    y = gen.GENERATORS_TORCH[args.kind](n, seed=2)
+    ws = pkg.Workspace(n)
+
+    # error bound: REL over the union range of both operands (all ranks must share one eb)
+    mm = torch.empty(4, dtype=torch.float32, device="cuda")
+    ws.value_range(x, mm[0:2])
+    ws.value_range(y, mm[2:4])
+    r = mm.cpu().numpy()
+    vmin, vmax = float(min(r[0], r[2])), float(max(r[1], r[3]))
+    eb = float(args.abs) if args.abs is not None else pkg.rel_to_abs(args.rel, vmin, vmax)
+
+    cap = pkg.max_stream_bytes(n)
+    cmp_a = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    cmp_b = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    cmp_s = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    dec = torch.empty(n, dtype=torch.float32, device="cuda")
+
+    ws.compress(x, eb, cmp_a)
+    la = ws.last_size()
+    ws.compress(y, eb, cmp_b)
+    lb = ws.last_size()
+    ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s)
+    ls = ws.last_size()
+
+    def step():
+        ws.compress(x, eb, cmp_a)
+        ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = 2 * 4 * n / (ms_per_step * 1e-3) / 1e9
+
+    # per-operation kernel times and roofline fractions (algorithmic bytes / time / HBM peak)
+    it = max(5, args.steps)
+    ops = {}
+
+    def add(name, fn, alg_bytes):
+        ms = time_op(torch, fn, it)
+        ops[name] = {"ms": round(ms, 4), "GBps_input": round(4 * n / ms / 1e6, 1),
+                     "alg_bytes": int(alg_bytes),
+                     "achieved_GBps": round(alg_bytes / ms / 1e6, 1),
+                     "frac_hbm": round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)}
+
+    add("compress", lambda: ws.compress(x, eb, cmp_a), 4 * n + la)
+    add("hom_sum_f32", lambda: ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s), la + 4 * n + ls)
+    add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n)
+    add("hom_add", lambda: ws.hom_add(cmp_a, la, cmp_b, lb, n, cmp_s), la + lb + ls)
+    torch.cuda.synchronize()
+
+    dom = "hom_sum_f32"
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": ops[dom]["achieved_GBps"],
+                "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ops[dom]["frac_hbm"],
+                "traffic": None}
+
+    out = {
+        "metric": "compress + hom-add throughput (GB/s of uncompressed input)",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32->i32", "data": "synthetic",
+        "config": {"workload": f"{args.kind} float32, 2^{args.log2n} elements per operand "
+                               f"({4 * n / 2**30:.2f} GiB), "
+                               + (f"ABS eb {eb:g}" if args.abs is not None else f"REL eb {args.rel:g} (abs {eb:.4g})")
+                               + ", step = compress(x) + hom_sum_f32(stream, y)",
+                   "elements": n, "eb_abs": eb},
+        "compression_ratio": round(4 * n / la, 3),
+        "compression_ratio_ref_convention": round(4 * n / pkg.ref_cmpsize(la, n), 3),
+        "compression_ratio_sum": round(4 * n / ls, 3),
+        "pct_hbm_peak": {k: round(100 * v["frac_hbm"], 2) for k, v in ops.items()},
+        "ops": ops,
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu:
+        orc = entry.load_oracle()
+        m = min(n, 1 << args.cpu_sample_log2)
+        xs, ys = x[:m].cpu().numpy(), y[:m].cpu().numpy()
+        base, sa, ss = cpu_baseline(orc, xs, ys, np.float32(eb))
+        # the sample doubles as a parity check of the two timed kernels
+        ga = torch.empty(pkg.max_stream_bytes(m), dtype=torch.uint8, device="cuda")
+        gs = torch.empty(pkg.max_stream_bytes(m), dtype=torch.uint8, device="cuda")
+        ws.compress(x[:m], eb, ga)
+        l1 = ws.last_size()
+        ws.hom_sum_f32(ga, l1, y[:m], eb, gs)
+        l2 = ws.last_size()
+        ok = (l1 == sa.size and l2 == ss.size
+              and np.array_equal(ga[:l1].cpu().numpy(), sa) and np.array_equal(gs[:l2].cpu().numpy(), ss))
+        base["gpu_matches_oracle_on_sample"] = bool(ok)
+        out["cpu_baseline"] = base
+        if not ok:
+            print(json.dumps(out))
+            print("GPU streams differ from the oracle on the sample", file=sys.stderr)
+            return 1
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
