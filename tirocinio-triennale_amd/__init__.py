@@ -42,6 +42,10 @@ def lib() -> C.CDLL:
             raise FileNotFoundError(
                 f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
                 f"(python tirocinio-triennale_amd/build.py)")
+        # torch ships its own HIP runtime and publishes it process-wide.  It has to be loaded
+        # before this library so that both bind to the same runtime instance: device pointers
+        # and hipStream_t handles are only meaningful inside the runtime that created them.
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         vp, sz, u64p = C.c_void_p, C.c_size_t, C.c_void_p
         L.homcomp_status_string.argtypes = [C.c_int]
