@@ -6,7 +6,7 @@ Two families of generators with the same shapes:
   from + - * only), so a given (kind, n, seed) is bit-identical on every machine.  Used for the
   committed golden fixtures and for CPU-sized parity cases.
 * ``*_torch`` -- the same formulae evaluated with torch on the GPU for the large benchmark
-  shapes (2^26 .. 2^28 elements); values are checked against the CPU oracle on the very same
+  shapes (2^26 .. 2^28 elements); their codec results are verified on the very same
   buffer, so they need not be bit-identical to the numpy family.
 
 Shapes (the three inputs the benchmark configurations name):
