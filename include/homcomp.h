@@ -41,6 +41,8 @@ extern "C" {
 #define HOMCOMP_ERR_TOO_LARGE (-3)    /* nbEle exceeds the workspace's max_nbEle                */
 #define HOMCOMP_ERR_HIP (-4)          /* a HIP runtime call failed; see homcomp_last_hip_error  */
 #define HOMCOMP_ERR_NO_DEVICE (-5)    /* no usable GPU                                           */
+#define HOMCOMP_ERR_SCAN_TIMEOUT (-6) /* a kernel gave up waiting in the offset scan (sticky);   */
+                                      /* streams produced since workspace creation are invalid   */
 
 typedef struct homcomp_workspace homcomp_workspace;
 
@@ -104,7 +106,8 @@ int homcomp_range_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, 
 float homcomp_rel_to_abs(float rel, float vmin, float vmax);
 
 /* The blocking read-back of src/GSZ_entry.cu:291 (cudaMemcpy of cmpOffset[gsize-1]): waits for
- * `stream` and returns the length L produced by the last stream-producing call on ws. */
+ * `stream` and returns the length L produced by the last stream-producing call on ws.  Also
+ * reports HOMCOMP_ERR_SCAN_TIMEOUT if any kernel on ws had to abandon its bounded wait. */
 int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream);
 
 #ifdef __cplusplus

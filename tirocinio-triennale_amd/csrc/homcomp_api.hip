@@ -15,6 +15,7 @@ namespace {
 thread_local int g_last_hip_error = 0;
 
 constexpr uint32_t kMaxEpoch = (1u << 22) - 1;
+constexpr uint32_t kSpinLimit = 1u << 22;   // unsuccessful scan probes (~seconds) before giving up
 constexpr uint32_t kRangePartials = 2048;
 
 inline bool hip_ok(hipError_t e)
@@ -35,14 +36,19 @@ struct homcomp_workspace {
     int device;
     size_t max_n;
     uint32_t max_tiles;
-    void *d_block;          // one allocation: status[3][max_tiles] | total | ticket | range partials
-    uint64_t *d_status[3];
-    uint64_t *d_total;
-    uint32_t *d_ticket;
-    float *d_partial;
-    uint64_t *h_total;      // pinned host word for the blocking size read-back
-    uint32_t epoch;         // last epoch handed out (1..kMaxEpoch)
-    uint32_t ticket_base;   // value of *d_ticket once all enqueued launches have run
+    uint32_t max_groups;
+    void *d_block;            // one allocation holding everything below
+    uint64_t *d_tile_status;  // [max_tiles]   output-offset scan, tile words
+    uint64_t *d_group_prefix; // [max_groups]  output-offset scan, group prefix words
+    uint64_t *d_group_acc;    // [max_groups * kHostAccStride]  output-offset scan, group accumulators
+    uint64_t *d_in_ofs[2];    // [max_tiles+1] tile payload offsets of the incoming streams
+    uint32_t *d_in_totals;    // [max_tiles]   scratch of the offsets pre-pass
+    uint64_t *d_total;        // stream length of the last stream-producing call
+    uint32_t *d_error;        // sticky error flags, next to d_total
+    float *d_partial;         // min/max partials
+    uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
+    uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
+    uint32_t max_grid[hc::kOpCount];  // resident workgroups of each tile kernel on this device
 };
 
 namespace {
@@ -57,11 +63,12 @@ int check_ws(const homcomp_workspace *ws, size_t n)
     return HOMCOMP_OK;
 }
 
-// Fresh epoch for one launch; clears the status words when the 22-bit tag wraps.
+// Fresh epoch for one launch; clears the status words when the 22-bit tag wraps (the two
+// status arrays are adjacent).
 int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
 {
     if (ws->epoch >= kMaxEpoch) {
-        if (!hip_ok(hc::launch_fill_u64(ws->d_status[0], (uint64_t)ws->max_tiles * 3, s)))
+        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_status, (uint64_t)ws->max_tiles + ws->max_groups, s)))
             return HOMCOMP_ERR_HIP;
         ws->epoch = 0;
     }
@@ -75,12 +82,32 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
     p->n = n;
     p->hdr_bytes = homcomp_header_bytes(n);
     p->n_tiles = (uint32_t)(padded_len(n) / hc::kHostTileElems);
-    for (int c = 0; c < 3; ++c) p->status[c] = ws->d_status[c];
-    p->ticket = ws->d_ticket;
-    p->ticket_base = ws->ticket_base;
-    ws->ticket_base += p->n_tiles;
+    p->tile_status = ws->d_tile_status;
+    p->group_prefix = ws->d_group_prefix;
+    p->group_acc = ws->d_group_acc;
+    p->spin_limit = kSpinLimit;
+    p->error = ws->d_error;
     p->total = ws->d_total;
     return next_epoch(ws, s, &p->epoch);
+}
+
+// Offsets pre-pass for incoming stream c (header bytes -> payload offset of every tile).
+int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::TileParams *p, hipStream_t s)
+{
+    p->in_ofs[c] = ws->d_in_ofs[c];
+    return hip_ok(hc::launch_in_offsets(d_cmp, p->n_tiles, p->hdr_bytes, ws->d_in_totals, ws->d_in_ofs[c], s))
+               ? HOMCOMP_OK
+               : HOMCOMP_ERR_HIP;
+}
+
+int run_tile_op(homcomp_workspace *ws, int op, const hc::TileParams &p, hipStream_t s)
+{
+    if (op != hc::kOpDecompress) {
+        // the group accumulators of the output-offset scan start every call at zero
+        const uint64_t groups = (p.n_tiles + hc::kHostGroupTiles - 1) / hc::kHostGroupTiles;
+        if (!hip_ok(hc::launch_fill_u64(ws->d_group_acc, groups * hc::kHostAccStride, s))) return HOMCOMP_ERR_HIP;
+    }
+    return hip_ok(hc::launch_tile_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
 // n == 0: the stream is empty; only the length words are written.
@@ -104,6 +131,7 @@ const char *homcomp_status_string(int status)
     case HOMCOMP_ERR_TOO_LARGE: return "nbEle exceeds the workspace capacity";
     case HOMCOMP_ERR_HIP: return "HIP runtime error";
     case HOMCOMP_ERR_NO_DEVICE: return "no usable GPU";
+    case HOMCOMP_ERR_SCAN_TIMEOUT: return "offset scan gave up waiting (grid not fully resident?); output invalid";
     default: return "unknown status";
     }
 }
@@ -147,19 +175,42 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
-    const size_t status_bytes = (size_t)ws->max_tiles * 3 * sizeof(uint64_t);
-    const size_t bytes = status_bytes + 256 + kRangePartials * 2 * sizeof(float);
-    if (!hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
-        !hip_ok(hipHostMalloc((void **)&ws->h_total, sizeof(uint64_t), hipHostMallocDefault))) {
+    ws->max_groups = (ws->max_tiles + hc::kHostGroupTiles - 1) / hc::kHostGroupTiles;
+    const size_t t = ws->max_tiles, g = ws->max_groups;
+    size_t off = 0;
+    auto take = [&off](size_t bytes) { size_t o = off; off = (off + bytes + 255) & ~(size_t)255; return o; };
+    const size_t o_status = take((t + g) * sizeof(uint64_t));
+    const size_t o_acc = take(g * hc::kHostAccStride * sizeof(uint64_t));
+    const size_t o_in0 = take((t + 1) * sizeof(uint64_t));
+    const size_t o_in1 = take((t + 1) * sizeof(uint64_t));
+    const size_t o_tot = take(t * sizeof(uint32_t));
+    const size_t o_total = take(64);
+    const size_t o_partial = take(kRangePartials * 2 * sizeof(float));
+    const size_t bytes = off;
+    hipDeviceProp_t prop;
+    bool ok = hip_ok(hipGetDeviceProperties(&prop, ws->device));
+    for (int op = 0; ok && op < hc::kOpCount; ++op) {
+        int per_cu = 0;
+        ok = hip_ok(hc::tile_kernel_residency(op, &per_cu));
+        if (ok && per_cu < 1) per_cu = 1;
+        ws->max_grid[op] = (uint32_t)per_cu * (uint32_t)prop.multiProcessorCount;
+    }
+    if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
+        !hip_ok(hipHostMalloc((void **)&ws->h_total, 2 * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
     uint8_t *base = (uint8_t *)ws->d_block;
-    for (int c = 0; c < 3; ++c) ws->d_status[c] = (uint64_t *)base + (size_t)c * ws->max_tiles;
-    ws->d_total = (uint64_t *)(base + status_bytes);
-    ws->d_ticket = (uint32_t *)(base + status_bytes + 128);
-    ws->d_partial = (float *)(base + status_bytes + 256);
+    ws->d_tile_status = (uint64_t *)(base + o_status);
+    ws->d_group_prefix = ws->d_tile_status + t;
+    ws->d_group_acc = (uint64_t *)(base + o_acc);
+    ws->d_in_ofs[0] = (uint64_t *)(base + o_in0);
+    ws->d_in_ofs[1] = (uint64_t *)(base + o_in1);
+    ws->d_in_totals = (uint32_t *)(base + o_tot);
+    ws->d_total = (uint64_t *)(base + o_total);
+    ws->d_error = (uint32_t *)(base + o_total + 8);
+    ws->d_partial = (float *)(base + o_partial);
     *out = ws;
     return HOMCOMP_OK;
 }
@@ -192,7 +243,7 @@ int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEl
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    return hip_ok(hc::launch_compress(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    return run_tile_op(ws, hc::kOpCompress, p, s);
 }
 
 int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
@@ -212,7 +263,8 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
     p.out_f32 = d_out;
     p.eb = eb;
     p.recip = 0.5f / eb;
-    return hip_ok(hc::launch_decompress(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    if ((rc = in_offsets(ws, 0, d_cmp, &p, s))) return rc;
+    return run_tile_op(ws, hc::kOpDecompress, p, s);
 }
 
 int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
@@ -235,7 +287,8 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    return hip_ok(hc::launch_hom_sum_f32(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
+    return run_tile_op(ws, hc::kOpHomSumF32, p, s);
 }
 
 int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
@@ -255,7 +308,8 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.local = d_local_delta;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    return hip_ok(hc::launch_hom_sum_i32(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
+    return run_tile_op(ws, hc::kOpHomSumI32, p, s);
 }
 
 int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t size_a,
@@ -275,7 +329,9 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
     p.in_size[1] = size_b;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    return hip_ok(hc::launch_hom_add(p, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    if ((rc = in_offsets(ws, 0, d_cmp_a, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, d_cmp_b, &p, s))) return rc;
+    return run_tile_op(ws, hc::kOpHomAdd, p, s);
 }
 
 int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,
@@ -307,11 +363,11 @@ int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream)
 {
     if (!ws || !stream_len) return HOMCOMP_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    if (!hip_ok(hipMemcpyAsync(ws->h_total, ws->d_total, sizeof(uint64_t), hipMemcpyDeviceToHost, s)) ||
+    if (!hip_ok(hipMemcpyAsync(ws->h_total, ws->d_total, 2 * sizeof(uint64_t), hipMemcpyDeviceToHost, s)) ||
         !hip_ok(hipStreamSynchronize(s)))
         return HOMCOMP_ERR_HIP;
-    *stream_len = (size_t)*ws->h_total;
-    return HOMCOMP_OK;
+    *stream_len = (size_t)ws->h_total[0];
+    return (uint32_t)ws->h_total[1] ? HOMCOMP_ERR_SCAN_TIMEOUT : HOMCOMP_OK;
 }
 
 }  // extern "C"

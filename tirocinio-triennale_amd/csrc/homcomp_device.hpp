@@ -22,7 +22,27 @@ constexpr int kTileBlocks = kBlocksPerIter * kIter;   // 128
 constexpr int kTileElems = kTileBlocks * 32;          // 4096
 constexpr int kChunkElems = 32768;                    // reference thread-block share
 constexpr int kMaxBlockBytes = 132;                   // largest size a header byte can imply
-constexpr int kStageBytes = kTileBlocks * kMaxBlockBytes + 64;
+constexpr int kStageBytes = kTileBlocks * kMaxBlockBytes + 64;      // LDS stage of an incoming tile
+constexpr int kOutBlockBytes = 128;                   // largest payload the encoder emits per block
+constexpr int kOutStageBytes = kTileBlocks * kOutBlockBytes + 64;   // LDS stage of an outgoing tile
+
+// Native 16-byte vectors (the streaming load/store builtins take these, not HIP's float4).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Every buffer is read or written exactly once per call, so loads and stores carry the
+// non-temporal hint and do not displace the scan words from the caches.
+template <typename V>
+__device__ __forceinline__ V stream_load(const void *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+}
+template <typename V>
+__device__ __forceinline__ void stream_store(void *p, V v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+}
 
 // ---------------------------------------------------------------- cross-lane helpers
 
@@ -242,15 +262,44 @@ __device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uin
     }
 }
 
-// ---------------------------------------------------------------- tile status words
+// ---------------------------------------------------------------- output-offset scan
 //
-// One 64-bit word per tile and scan chain: bits 63-62 state (0 empty, 1 tile aggregate,
-// 2 inclusive prefix), bits 61-40 the call's epoch, bits 39-0 the byte count.  A word whose
-// epoch is not the current call's reads as empty, so the array never needs clearing between
-// calls (the host clears it when the 22-bit epoch wraps).
+// The byte offset of a tile's payload in the outgoing stream is an exclusive prefix sum over
+// all earlier tiles (HomComp/src/GSZ.cu:170-239).  It is resolved in a single pass, without any
+// workgroup ever having to wait for another one in the steady state:
+//
+//   publish   (round i)    the tile stores its byte total in its tile word and adds it, together
+//                          with a count of one, to the accumulator word of its group of 64 tiles
+//                          (a fire-and-forget atomic);
+//   probe     (round i+1)  the tile's wave issues the loads of: the tile words of the earlier
+//                          tiles of its group, and for the 64 groups before its own the
+//                          accumulator word and the prefix word;
+//   resolve   (round i+2)  the loaded words are a round old and were published two rounds ago:
+//                          exclusive prefix = (nearest published group prefix) + (accumulators of
+//                          the complete groups after it) + (tile words of the group's earlier
+//                          tiles).  The last tile of a group publishes the group's prefix word.
+//
+// Tile and prefix words carry an epoch tag: bits 63-62 state (0 empty, 1 tile total, 2 inclusive
+// group prefix), bits 61-40 the call's epoch, bits 39-0 a byte count; a word of another epoch
+// reads as empty, so these arrays are never cleared between calls (the host clears them when the
+// 22-bit epoch wraps).  Accumulator words (bits 39-32 count, bits 31-0 byte sum) are zeroed
+// before every call.
+//
+// All tiles with a smaller index are processed by workgroups that are resident at the same time
+// (the grid is sized to fit the device), so a missing word is always on its way; if a probe does
+// come back incomplete the wave re-reads until it is complete.  As a guard against a launch that
+// could not become fully resident these waits are bounded: after `spin_limit` unsuccessful
+// re-reads the wave raises *err and goes on with what it has, so the kernel always terminates.
 
 constexpr uint64_t kValueMask = (1ull << 40) - 1;
 constexpr uint32_t kEpochMask = (1u << 22) - 1;
+constexpr int kGroupShift = 6;   // 64 tiles per group
+constexpr uint32_t kGroupMask = (1u << kGroupShift) - 1u;
+constexpr uint32_t kGroupFull = 1u << kGroupShift;
+// Read-modify-write atomics that hit one cache line are serialised by the memory side (about
+// 11 ns each on MI355X, measured), whichever word of the line they address; the accumulators of
+// the groups in flight are updated at the same time, so each gets a 128-byte line of its own.
+constexpr int kAccStride = 16;   // 64-bit words between two accumulators
 
 __device__ __forceinline__ uint64_t status_word(uint32_t epoch, uint32_t state, uint64_t value)
 {
@@ -267,42 +316,111 @@ __device__ __forceinline__ void status_store(uint64_t *p, uint64_t w)
     __hip_atomic_store(p, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Decoupled look-back over the tile status words, run by one full wave.  Publishes this
-// tile's aggregate, sums the aggregates of the predecessors back to the nearest published
-// inclusive prefix (64 predecessors per probe), publishes this tile's inclusive prefix and
-// returns its exclusive prefix.  Tiles take their index from a ticket counter, so every
-// predecessor is already running when a tile starts to wait.
-__device__ __forceinline__ uint64_t lookback(uint64_t *status, uint32_t tile, uint32_t epoch,
-                                             uint64_t aggregate, int lane)
+// state of a word under the current epoch (0 when the word belongs to an earlier call)
+__device__ __forceinline__ uint32_t status_state(uint64_t w, uint32_t epoch)
 {
-    if (tile == 0) {
-        if (lane == 0) status_store(&status[0], status_word(epoch, 2, aggregate));
-        return 0;
+    return (((uint32_t)(w >> 40)) & kEpochMask) == (epoch & kEpochMask) ? (uint32_t)(w >> 62) : 0u;
+}
+
+struct ScanCtx {
+    uint64_t *tstat;   // tile words
+    uint64_t *gacc;    // group accumulators (zero when the call starts), kAccStride words apart
+    uint64_t *gpref;   // group prefix words
+    uint32_t n_tiles;
+    uint32_t epoch;
+    uint32_t spin_limit;
+    uint32_t *err;
+};
+
+struct ScanProbe {
+    uint64_t wt;   // lane l: tile word of the l-th tile of the group (l < position in group)
+    uint64_t wa;   // lane l: accumulator of group (first - l)
+    uint64_t wp;   // lane l: prefix word of group (first - l)
+};
+
+__device__ __forceinline__ void scan_publish(const ScanCtx &c, uint32_t tile, uint32_t total, int lane)
+{
+    if (lane == 0) {
+        status_store(&c.tstat[tile], status_word(c.epoch, 1, total));
+        (void)__hip_atomic_fetch_add(&c.gacc[(uint64_t)(tile >> kGroupShift) * kAccStride],
+                                     (1ull << 32) | (uint64_t)total,
+                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (lane == 0) status_store(&status[tile], status_word(epoch, 1, aggregate));
-    uint64_t excl = 0;
-    int64_t base = (int64_t)tile - 1;
+}
+
+__device__ __forceinline__ uint64_t scan_probe_tiles(const ScanCtx &c, uint32_t tile, int lane)
+{
+    return (uint32_t)lane < (tile & kGroupMask) ? status_load(&c.tstat[(tile & ~kGroupMask) + lane]) : 0ull;
+}
+
+__device__ __forceinline__ void scan_probe_groups(const ScanCtx &c, int64_t first, int lane,
+                                                  uint64_t &wa, uint64_t &wp)
+{
+    const int64_t gi = first - lane;
+    wa = 0;
+    wp = 0;
+    if (gi >= 0) {
+        wa = status_load(&c.gacc[gi * kAccStride]);
+        wp = status_load(&c.gpref[gi]);
+    }
+}
+
+__device__ __forceinline__ ScanProbe scan_probe(const ScanCtx &c, uint32_t tile, int lane)
+{
+    ScanProbe pr;
+    pr.wt = scan_probe_tiles(c, tile, lane);
+    scan_probe_groups(c, (int64_t)(tile >> kGroupShift) - 1, lane, pr.wa, pr.wp);
+    return pr;
+}
+
+__device__ __forceinline__ bool scan_give_up(const ScanCtx &c, uint32_t &spins, int lane)
+{
+    if (++spins > c.spin_limit) {
+        if (lane == 0) atomicOr(c.err, 1u);
+        return true;
+    }
+    __builtin_amdgcn_s_sleep(1);
+    return false;
+}
+
+// Exclusive prefix of `tile` from an earlier scan_probe(tile); run by one full wave.
+__device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint32_t total,
+                                                 ScanProbe pr, int lane)
+{
+    const uint32_t g = tile >> kGroupShift;
+    const uint32_t r = tile & kGroupMask;
+    uint32_t spins = 0;
+    // earlier tiles of the same group
+    while (__ballot((uint32_t)lane < r && status_state(pr.wt, c.epoch) == 0) != 0) {
+        if (scan_give_up(c, spins, lane)) break;
+        pr.wt = scan_probe_tiles(c, tile, lane);
+    }
+    uint64_t excl = wave_sum_u64((uint32_t)lane < r ? (pr.wt & kValueMask) : 0ull);
+    // earlier groups: back to the nearest published prefix
+    int64_t first = (int64_t)g - 1;
     for (;;) {
-        const int64_t idx = base - lane;
-        uint64_t w = 0;
-        uint32_t st = 2;                                  // virtual zero prefix before tile 0
-        if (idx >= 0) {
-            w = status_load(&status[idx]);
-            st = (((uint32_t)(w >> 40)) & kEpochMask) == (epoch & kEpochMask) ? (uint32_t)(w >> 62) : 0u;
-        }
-        const uint64_t m_empty = __ballot(st == 0);
-        const uint64_t m_prefix = __ballot(st == 2);
-        const int first = m_prefix ? __builtin_ctzll(m_prefix) : 63;
-        const uint64_t need = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
-        if (m_empty & need) {
-            __builtin_amdgcn_s_sleep(2);
+        const int64_t gi = first - lane;
+        const bool has_prefix = gi < 0 || status_state(pr.wp, c.epoch) == 2u;   // zero prefix before group 0
+        const bool complete = gi >= 0 && (uint32_t)((pr.wa >> 32) & 0xffu) == kGroupFull;
+        const uint64_t m_prefix = __ballot(has_prefix);
+        const uint64_t m_open = __ballot(!has_prefix && !complete);
+        const int stop = m_prefix ? __builtin_ctzll(m_prefix) : 64;
+        const uint64_t before = stop >= 64 ? ~0ull : ((1ull << stop) - 1ull);   // lanes that must be complete
+        if (m_open & before) {
+            if (scan_give_up(c, spins, lane)) break;
+            scan_probe_groups(c, first, lane, pr.wa, pr.wp);
             continue;
         }
-        excl += wave_sum_u64(lane <= first ? (w & kValueMask) : 0ull);
+        uint64_t v = 0;
+        if (lane < stop) v = pr.wa & 0xffffffffull;
+        else if (lane == stop && gi >= 0) v = pr.wp & kValueMask;
+        excl += wave_sum_u64(v);
         if (m_prefix) break;
-        base -= 64;
+        first -= 64;
+        scan_probe_groups(c, first, lane, pr.wa, pr.wp);
     }
-    if (lane == 0) status_store(&status[tile], status_word(epoch, 2, excl + aggregate));
+    if (((tile & kGroupMask) == kGroupMask || tile == c.n_tiles - 1u) && lane == 0)
+        status_store(&c.gpref[g], status_word(c.epoch, 2, excl + total));
     return excl;
 }
 

@@ -1,16 +1,24 @@
-// HomComp kernels for gfx950: one tiled, single-pass kernel template covers compress,
-// decompress and the three homomorphic sums; two small streaming kernels cover the Lorenzo
-// pre-pass and the value range.
+// HomComp kernels for gfx950.
 //
-// A tile is 4096 elements = 128 blocks, processed by one 256-thread workgroup in two
-// iterations of 8 elements per lane.  Phases of the tile kernel:
-//   1. take a tile index from the ticket counter; start the loads of the local operand
-//   2. per incoming stream: header bytes -> block sizes -> tile-local scan -> look-back for the
-//      tile's payload offset -> coalesced 16-byte copy of the payload into LDS -> per-lane decode
-//   3. combine: delta_out = delta_local + sum of decoded deltas (HomComp/src/homcomp.cu:3611-3616)
-//   4a. stream output: rate selection, header bytes, tile-local scan, look-back on the output
-//       chain (overlapped with packing into LDS), coalesced 16-byte copy to the stream
+// k_tile<NIN, LOCAL, OUT> is one persistent, tiled, single-pass kernel template that covers
+// compress, decompress and the three homomorphic sums.  A tile is 4096 elements = 128 blocks,
+// processed by one 256-thread workgroup in two iterations of 8 elements per lane.  The grid is
+// sized to what the device can keep resident and walks the tiles in rounds
+// (tile = blockIdx.x, += gridDim.x), so the loads of the next tile are issued while the
+// current one is still being packed and stored.  Phases per tile:
+//   1. local operand (float32 values or int32 deltas) -> registers (prefetched one tile ahead)
+//   2. per incoming stream: tile payload offset from the offsets array that k_in_totals /
+//      k_in_scan produced from the header bytes; header bytes -> block sizes -> tile-local
+//      scan; coalesced 16-byte copy of the payload into LDS; per-lane decode
+//   3. combine: delta_out = delta_local + decoded deltas (HomComp/src/homcomp.cu:3611-3616)
+//   4a. stream output: rate selection, header bytes, tile-local scan, pack into one of two LDS
+//       buffers; the tile's offset in the stream comes from a two-level single-pass scan whose
+//       steps (publish, probe, resolve) are spread over this and the next two rounds, so the
+//       payload is copied to the stream (coalesced 16-byte stores) two rounds after it was
+//       packed and no round waits for another workgroup
 //   4b. float output: in-block running sum, dequantise, two float4 stores per lane
+// Small streaming kernels cover the incoming-stream offsets, the Lorenzo pre-pass and the
+// value range.
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
@@ -28,235 +36,354 @@ __device__ __forceinline__ uint32_t tile_scan(const uint32_t *s_size, uint32_t *
     return __shfl(incl, 63, 64);
 }
 
+// Registers holding one tile's share of the local operand.
+template <int LOCAL>
+struct LocalRegs {
+    f32x4 f[kIter][2];
+    i32x4 i[kIter][2];
+};
+
+template <int LOCAL>
+__device__ __forceinline__ void load_local(LocalRegs<LOCAL> &r, const void *local, uint64_t n,
+                                           uint64_t tile_elem0, int tid)
+{
+    if constexpr (LOCAL == kLocalNone) return;
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+        const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
+        if (e0 + kEPL <= n) {
+            if constexpr (LOCAL == kLocalF32) {
+                const float *src = (const float *)local + e0;
+                r.f[it][0] = stream_load<f32x4>(src);
+                r.f[it][1] = stream_load<f32x4>(src + 4);
+            } else {
+                const int32_t *src = (const int32_t *)local + e0;
+                r.i[it][0] = stream_load<i32x4>(src);
+                r.i[it][1] = stream_load<i32x4>(src + 4);
+            }
+        } else {
+            float tf[8];
+            int32_t ti[8];
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                const bool in = e0 + m < n;
+                if constexpr (LOCAL == kLocalF32)
+                    tf[m] = in ? ((const float *)local)[e0 + m] : 0.0f;
+                else
+                    ti[m] = in ? ((const int32_t *)local)[e0 + m] : 0;
+            }
+            if constexpr (LOCAL == kLocalF32) {
+                r.f[it][0] = f32x4{tf[0], tf[1], tf[2], tf[3]};
+                r.f[it][1] = f32x4{tf[4], tf[5], tf[6], tf[7]};
+            } else {
+                r.i[it][0] = i32x4{ti[0], ti[1], ti[2], ti[3]};
+                r.i[it][1] = i32x4{ti[4], ti[5], ti[6], ti[7]};
+            }
+        }
+    }
+}
+
+// Coalesced copy of a packed tile payload from LDS to its (arbitrarily aligned) place in the
+// stream: bytes up to the first 16-byte boundary, aligned 16-byte stores assembled from
+// unaligned LDS words with v_alignbyte, then the remaining bytes.
+__device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint32_t tot, int tid)
+{
+    const uint32_t mis = (uint32_t)((uintptr_t)g & 15u);
+    uint32_t head = (16u - mis) & 15u;
+    if (head > tot) head = tot;
+    const uint32_t body = tot - head;
+    const uint32_t nch = body >> 4;
+    const uint32_t tail = body & 15u;
+    if ((uint32_t)tid < head) g[tid] = stage[tid];
+    const uint32_t *sw = reinterpret_cast<const uint32_t *>(stage);
+    for (uint32_t c = tid; c < nch; c += kWG) {
+        const uint32_t s = head + 16u * c;
+        const uint32_t w0 = s >> 2, sh = s & 3u;
+        const uint32_t x0 = sw[w0], x1 = sw[w0 + 1], x2 = sw[w0 + 2], x3 = sw[w0 + 3], x4 = sw[w0 + 4];
+        u32x4 o;
+        o.x = __builtin_amdgcn_alignbyte(x1, x0, sh);
+        o.y = __builtin_amdgcn_alignbyte(x2, x1, sh);
+        o.z = __builtin_amdgcn_alignbyte(x3, x2, sh);
+        o.w = __builtin_amdgcn_alignbyte(x4, x3, sh);
+        stream_store<u32x4>(g + s, o);
+    }
+    if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = stage[head + 16u * nch + tid];
+}
+
 template <int NIN, int LOCAL, int OUT>
 __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
 {
-    constexpr int kStages = NIN > 1 ? NIN : 1;
-    __shared__ __align__(16) uint8_t s_stage[kStages][kStageBytes];
+    constexpr bool kEnc = OUT == kOutStream;
+    constexpr int kIn = NIN > 0 ? NIN : 1;
+    __shared__ __align__(16) uint8_t s_in[kIn][NIN > 0 ? kStageBytes : 16];
+    __shared__ __align__(16) uint8_t s_out[2][kEnc ? kOutStageBytes : 16];
     __shared__ uint32_t s_size[kTileBlocks];
-    __shared__ uint32_t s_ofs[kStages][kTileBlocks];
-    __shared__ uint8_t s_hdr[kStages][kTileBlocks];
-    __shared__ uint64_t s_base[kStages];
-    __shared__ uint32_t s_total[kStages];
-    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_ofs_in[kIn][kTileBlocks];
+    __shared__ uint32_t s_ofs_out[kTileBlocks];
+    __shared__ uint8_t s_hdr_in[kIn][kTileBlocks];
+    __shared__ uint8_t s_hdr_out[kTileBlocks];
+    __shared__ uint64_t s_base;
+    __shared__ uint32_t s_total;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int k = tid & 3;
     const int quad = tid >> 2;
+    const int64_t G = gridDim.x;
+    const int64_t n_tiles = p.n_tiles;
+    const ScanCtx scan{p.tile_status, p.group_acc, p.group_prefix, p.n_tiles, p.epoch, p.spin_limit, p.error};
 
-    if (tid == 0) s_tile = atomicAdd(p.ticket, 1u) - p.ticket_base;
-    __syncthreads();
-    const uint32_t tile = s_tile;
-    const uint64_t tile_elem0 = (uint64_t)tile * kTileElems;
+    LocalRegs<LOCAL> nxt;
+    if ((int64_t)blockIdx.x < n_tiles)
+        load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)blockIdx.x * kTileElems, tid);
 
-    // ---- local operand: issue the loads first so they fly during the stream bookkeeping
-    float4 lf[kIter][2];
-    int4 li[kIter][2];
-    if constexpr (LOCAL != kLocalNone) {
+    // scan pipeline registers of wave 0: byte totals of the tiles of the previous two rounds and
+    // the probe that was issued in the previous round for the older of the two
+    uint32_t total1 = 0, total2 = 0;
+    ScanProbe probe{0, 0, 0};
+
+    // Round i handles tile t0 = blockIdx.x + i*G and, on the encoder, finishes the scan and the
+    // store of the tiles of the two rounds before (t1, t2).
+    for (int64_t t0 = blockIdx.x;; t0 += G) {
+        const int64_t t1 = t0 - G, t2 = t0 - 2 * G;
+        const bool v0 = t0 < n_tiles;
+        const bool v1 = kEnc && t1 >= 0 && t1 < n_tiles;
+        const bool v2 = kEnc && t2 >= 0 && t2 < n_tiles;
+        if (!v0 && !v1 && !v2) break;
+        const uint32_t tile = (uint32_t)t0;
+        const int buf = (int)((t0 / G) & 1);
+
+        uint32_t a[kIter][8], sb[kIter], hd[kIter];
+        if (v0) {
+            const uint64_t tile_elem0 = (uint64_t)tile * kTileElems;
+
+            // ---- incoming streams: header bytes, block offsets, payload into LDS
+            uint64_t in_base[kIn];
+            uint32_t in_shift[kIn];
 #pragma unroll
-        for (int it = 0; it < kIter; ++it) {
-            const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
-            if (e0 + kEPL <= p.n) {
-                if constexpr (LOCAL == kLocalF32) {
-                    const float4 *src = reinterpret_cast<const float4 *>((const float *)p.local + e0);
-                    lf[it][0] = src[0];
-                    lf[it][1] = src[1];
-                } else {
-                    const int4 *src = reinterpret_cast<const int4 *>((const int32_t *)p.local + e0);
-                    li[it][0] = src[0];
-                    li[it][1] = src[1];
+            for (int c = 0; c < NIN; ++c) {
+                const uint64_t start = p.in_ofs[c][tile];
+                const uint32_t total = (uint32_t)(p.in_ofs[c][tile + 1] - start);
+                in_base[c] = start;
+                if (tid < kTileBlocks) {
+                    const uint32_t h = p.in[c][(uint64_t)tile * kTileBlocks + tid];
+                    s_hdr_in[c][tid] = (uint8_t)h;
+                    s_size[tid] = size_from_header(h);
                 }
+                const uintptr_t g0 = (uintptr_t)p.in[c] + start;
+                const uintptr_t ga = g0 & ~(uintptr_t)15;
+                const uint32_t shift = (uint32_t)(g0 - ga);
+                in_shift[c] = shift;
+                const uint32_t nbytes = total ? shift + total : 0u;
+                const uint32_t nchunks = (nbytes + 15u) >> 4;
+                for (uint32_t i = tid; i < nchunks; i += kWG) {
+                    if (16u * (i + 1u) <= nbytes) {
+                        *reinterpret_cast<u32x4 *>(&s_in[c][16u * i]) =
+                            stream_load<u32x4>(reinterpret_cast<const void *>(ga + 16u * (uintptr_t)i));
+                    } else {
+                        for (uint32_t j = 16u * i; j < nbytes; ++j)
+                            s_in[c][j] = *reinterpret_cast<const uint8_t *>(ga + j);
+                    }
+                }
+                __syncthreads();
+                if (wave == 0) tile_scan(s_size, s_ofs_in[c], lane);
+                __syncthreads();
+            }
+
+            // ---- per iteration: local deltas + decoded deltas
+            int32_t v[kIter][8];
+#pragma unroll
+            for (int it = 0; it < kIter; ++it) {
+                const int blk = it * kBlocksPerIter + quad;
+                if constexpr (LOCAL == kLocalF32) {
+                    // HomComp/src/GSZ.cu:82-149: quantise, Lorenzo with prevQuant = 0 at block start
+                    const float x[8] = {nxt.f[it][0].x, nxt.f[it][0].y, nxt.f[it][0].z, nxt.f[it][0].w,
+                                        nxt.f[it][1].x, nxt.f[it][1].y, nxt.f[it][1].z, nxt.f[it][1].w};
+                    int32_t q[8];
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) q[m] = quantize(x[m], p.recip);
+                    uint32_t prev = dpp_u32<kDppRowShr1>((uint32_t)q[7]);
+                    if (k == 0) prev = 0;
+                    v[it][0] = (int32_t)((uint32_t)q[0] - prev);
+#pragma unroll
+                    for (int m = 1; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)q[m] - (uint32_t)q[m - 1]);
+                } else if constexpr (LOCAL == kLocalI32) {
+                    // HomComp/src/homcomp.cu:2252-2268: precomputed deltas
+                    v[it][0] = nxt.i[it][0].x; v[it][1] = nxt.i[it][0].y; v[it][2] = nxt.i[it][0].z; v[it][3] = nxt.i[it][0].w;
+                    v[it][4] = nxt.i[it][1].x; v[it][5] = nxt.i[it][1].y; v[it][6] = nxt.i[it][1].z; v[it][7] = nxt.i[it][1].w;
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) v[it][m] = 0;
+                }
+#pragma unroll
+                for (int c = 0; c < NIN; ++c) {
+                    const uint32_t h = s_hdr_in[c][blk];
+                    const uint32_t ofs = s_ofs_in[c][blk];
+                    // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
+                    const bool active = size_from_header(h) != 0u && in_base[c] + ofs < p.in_size[c];
+                    int32_t d[8];
+                    unpack8(s_in[c], in_shift[c] + ofs, h, active, k, d);
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)v[it][m] + (uint32_t)d[m]);
+                }
+            }
+
+            // ---- the local operand of the next round starts to fly now
+            if (t0 + G < n_tiles)
+                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + G) * kTileElems, tid);
+
+            if constexpr (!kEnc) {
+                // ---- HomComp/src/GSZ.cu:1426-1468: running sum inside the block, dequantise, store
+#pragma unroll
+                for (int it = 0; it < kIter; ++it) {
+                    uint32_t q[8];
+                    q[0] = (uint32_t)v[it][0];
+#pragma unroll
+                    for (int m = 1; m < 8; ++m) q[m] = q[m - 1] + (uint32_t)v[it][m];
+                    const uint32_t s0 = dpp_u32<kDppBcast0>(q[7]);
+                    const uint32_t s1 = dpp_u32<kDppBcast1>(q[7]);
+                    const uint32_t s2 = dpp_u32<kDppBcast2>(q[7]);
+                    const uint32_t off = (k > 0 ? s0 : 0u) + (k > 1 ? s1 : 0u) + (k > 2 ? s2 : 0u);
+                    float y[8];
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) y[m] = dequantize((int32_t)(q[m] + off), p.eb);
+                    const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
+                    if (e0 + kEPL <= p.n) {
+                        float *dst = p.out_f32 + e0;
+                        stream_store<f32x4>(dst, f32x4{y[0], y[1], y[2], y[3]});
+                        stream_store<f32x4>(dst + 4, f32x4{y[4], y[5], y[6], y[7]});
+                    } else {
+#pragma unroll
+                        for (int m = 0; m < 8; ++m)
+                            if (e0 + m < p.n) p.out_f32[e0 + m] = y[m];
+                    }
+                }
+                __syncthreads();  // LDS of this tile is dead before the next round overwrites it
             } else {
-                float tf[8];
-                int32_t ti[8];
+                // ---- rate selection and header bytes (HomComp/src/GSZ.cu:151-167)
 #pragma unroll
-                for (int m = 0; m < 8; ++m) {
-                    const bool in = e0 + m < p.n;
-                    if constexpr (LOCAL == kLocalF32)
-                        tf[m] = in ? ((const float *)p.local)[e0 + m] : 0.0f;
-                    else
-                        ti[m] = in ? ((const int32_t *)p.local)[e0 + m] : 0;
+                for (int it = 0; it < kIter; ++it) {
+                    uint32_t size;
+                    analyse8(v[it], k, a[it], sb[it], hd[it], size);
+                    if (k == 0) {
+                        const int blk = it * kBlocksPerIter + quad;
+                        s_size[blk] = size;
+                        s_hdr_out[blk] = (uint8_t)hd[it];
+                    }
                 }
-                if constexpr (LOCAL == kLocalF32) {
-                    lf[it][0] = make_float4(tf[0], tf[1], tf[2], tf[3]);
-                    lf[it][1] = make_float4(tf[4], tf[5], tf[6], tf[7]);
-                } else {
-                    li[it][0] = make_int4(ti[0], ti[1], ti[2], ti[3]);
-                    li[it][1] = make_int4(ti[4], ti[5], ti[6], ti[7]);
+            }
+        }
+
+        if constexpr (kEnc) {
+            __syncthreads();
+            if (v0 && tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr_out[tid];
+            // ---- wave 0: tile-local scan and the scan steps (HomComp/src/GSZ.cu:170-239): publish
+            //      this round's tile, resolve the tile of two rounds ago from the probe issued in
+            //      the previous round, issue the probe for the previous round's tile
+            if (wave == 0) {
+                uint32_t total0 = 0;
+                if (v0) {
+                    total0 = tile_scan(s_size, s_ofs_out, lane);
+                    scan_publish(scan, tile, total0, lane);
+                }
+                if (v2) {
+                    const uint64_t excl = scan_resolve(scan, (uint32_t)t2, total2, probe, lane);
+                    if (lane == 0) {
+                        s_base = p.hdr_bytes + excl;
+                        s_total = total2;
+                    }
+                }
+                if (v1) probe = scan_probe(scan, (uint32_t)t1, lane);
+                total2 = total1;
+                total1 = total0;
+            }
+            __syncthreads();
+            // ---- the tile packed two rounds ago goes to its place in the stream
+            if (v2) {
+                const uint64_t gofs = s_base;
+                const uint32_t tot = s_total;
+                copy_out(s_out[buf], p.out_cmp + gofs, tot, tid);
+                // true stream length = end offset of the last tile (HomComp/src/GSZ.cu:752-755)
+                if (t2 == n_tiles - 1 && tid == 0) {
+                    const uint64_t len = gofs + tot;
+                    *p.total = len;
+                    if (p.user_total) *p.user_total = len;
+                }
+            }
+            __syncthreads();
+            // ---- and this round's tile takes over the buffer (HomComp/src/GSZ.cu:241-751)
+            if (v0) {
+#pragma unroll
+                for (int it = 0; it < kIter; ++it) {
+                    const int blk = it * kBlocksPerIter + quad;
+                    pack8(s_out[buf], s_ofs_out[blk], hd[it], k, a[it], sb[it]);
                 }
             }
         }
     }
+}
 
-    // ---- incoming streams: sizes, offsets, payload into LDS
-    uint32_t in_shift[kStages];
-#pragma unroll
-    for (int c = 0; c < NIN; ++c) {
-        if (tid < kTileBlocks) {
-            const uint32_t h = p.in[c][(uint64_t)tile * kTileBlocks + tid];
-            s_hdr[c][tid] = (uint8_t)h;
-            s_size[tid] = size_from_header(h);
-        }
-        __syncthreads();
-        if (wave == 0) {
-            const uint32_t total = tile_scan(s_size, s_ofs[c], lane);
-            const uint64_t excl = lookback(p.status[c], tile, p.epoch, total, lane);
-            if (lane == 0) {
-                s_base[c] = p.hdr_bytes + excl;
-                s_total[c] = total;
-            }
-        }
-        __syncthreads();
-        const uint64_t start = s_base[c];
-        const uint32_t total = s_total[c];
-        const uintptr_t g0 = (uintptr_t)p.in[c] + start;
-        const uintptr_t ga = g0 & ~(uintptr_t)15;
-        const uint32_t shift = (uint32_t)(g0 - ga);
-        in_shift[c] = shift;
-        const uint32_t nbytes = total ? shift + total : 0u;
-        const uint32_t nchunks = (nbytes + 15u) >> 4;
-        for (uint32_t i = tid; i < nchunks; i += kWG) {
-            if (16u * (i + 1u) <= nbytes) {
-                *reinterpret_cast<uint4 *>(&s_stage[c][16u * i]) =
-                    *reinterpret_cast<const uint4 *>(ga + 16u * (uintptr_t)i);
-            } else {
-                for (uint32_t j = 16u * i; j < nbytes; ++j)
-                    s_stage[c][j] = *reinterpret_cast<const uint8_t *>(ga + j);
-            }
-        }
-        __syncthreads();
-    }
+// ---------------------------------------------------------------- incoming-stream offsets
+//
+// The payload offset of a tile of an incoming stream depends on the header bytes only
+// (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel: k_in_totals sums
+// the block sizes of every tile (8 lanes per tile, 16 header bytes per lane), k_in_scan turns
+// the totals into exclusive offsets (one workgroup; `base` = header length is added).
 
-    // ---- per iteration: local deltas + decoded deltas
-    int32_t v[kIter][8];
-#pragma unroll
-    for (int it = 0; it < kIter; ++it) {
-        const int blk = it * kBlocksPerIter + quad;
-        if constexpr (LOCAL == kLocalF32) {
-            // HomComp/src/GSZ.cu:82-149: quantise, then Lorenzo with prevQuant = 0 at block start
-            const float x[8] = {lf[it][0].x, lf[it][0].y, lf[it][0].z, lf[it][0].w,
-                                lf[it][1].x, lf[it][1].y, lf[it][1].z, lf[it][1].w};
-            int32_t q[8];
-#pragma unroll
-            for (int m = 0; m < 8; ++m) q[m] = quantize(x[m], p.recip);
-            uint32_t prev = dpp_u32<kDppRowShr1>((uint32_t)q[7]);
-            if (k == 0) prev = 0;
-            v[it][0] = (int32_t)((uint32_t)q[0] - prev);
-#pragma unroll
-            for (int m = 1; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)q[m] - (uint32_t)q[m - 1]);
-        } else if constexpr (LOCAL == kLocalI32) {
-            // HomComp/src/homcomp.cu:2252-2268: precomputed deltas
-            v[it][0] = li[it][0].x; v[it][1] = li[it][0].y; v[it][2] = li[it][0].z; v[it][3] = li[it][0].w;
-            v[it][4] = li[it][1].x; v[it][5] = li[it][1].y; v[it][6] = li[it][1].z; v[it][7] = li[it][1].w;
+__global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ hdr, uint32_t n_tiles,
+                                                   uint32_t *__restrict__ totals)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;   // 16-byte piece index
+    const uint32_t tile = t >> 3;
+    uint32_t sum = 0;
+    if (tile < n_tiles) {
+        const uint8_t *src = hdr + (uint64_t)t * 16u;
+        uint32_t w[4];
+        if (((uintptr_t)src & 15u) == 0) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(src);
+            w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
         } else {
 #pragma unroll
-            for (int m = 0; m < 8; ++m) v[it][m] = 0;
+            for (int i = 0; i < 4; ++i)
+                w[i] = (uint32_t)src[4 * i] | ((uint32_t)src[4 * i + 1] << 8) |
+                       ((uint32_t)src[4 * i + 2] << 16) | ((uint32_t)src[4 * i + 3] << 24);
         }
 #pragma unroll
-        for (int c = 0; c < NIN; ++c) {
-            const uint32_t h = s_hdr[c][blk];
-            const uint32_t ofs = s_ofs[c][blk];
-            // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
-            const bool active = size_from_header(h) != 0u && s_base[c] + ofs < p.in_size[c];
-            int32_t d[8];
-            unpack8(s_stage[c], in_shift[c] + ofs, h, active, k, d);
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int m = 0; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)v[it][m] + (uint32_t)d[m]);
-        }
+            for (int b = 0; b < 4; ++b) sum += size_from_header((w[i] >> (8 * b)) & 0xffu);
     }
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    if (tile < n_tiles && (threadIdx.x & 7) == 0) totals[tile] = sum;
+}
 
-    if constexpr (OUT == kOutF32) {
-        // ---- HomComp/src/GSZ.cu:1426-1468: running sum inside the block, dequantise, store
-#pragma unroll
-        for (int it = 0; it < kIter; ++it) {
-            uint32_t q[8];
-            q[0] = (uint32_t)v[it][0];
-#pragma unroll
-            for (int m = 1; m < 8; ++m) q[m] = q[m - 1] + (uint32_t)v[it][m];
-            const uint32_t t0 = dpp_u32<kDppBcast0>(q[7]);
-            const uint32_t t1 = dpp_u32<kDppBcast1>(q[7]);
-            const uint32_t t2 = dpp_u32<kDppBcast2>(q[7]);
-            const uint32_t off = (k > 0 ? t0 : 0u) + (k > 1 ? t1 : 0u) + (k > 2 ? t2 : 0u);
-            float y[8];
-#pragma unroll
-            for (int m = 0; m < 8; ++m) y[m] = dequantize((int32_t)(q[m] + off), p.eb);
-            const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
-            if (e0 + kEPL <= p.n) {
-                float4 *dst = reinterpret_cast<float4 *>(p.out_f32 + e0);
-                dst[0] = make_float4(y[0], y[1], y[2], y[3]);
-                dst[1] = make_float4(y[4], y[5], y[6], y[7]);
-            } else {
-#pragma unroll
-                for (int m = 0; m < 8; ++m)
-                    if (e0 + m < p.n) p.out_f32[e0 + m] = y[m];
-            }
-        }
-    } else {
-        // ---- rate selection and header bytes (HomComp/src/GSZ.cu:151-167)
-        uint32_t a[kIter][8], sb[kIter], hd[kIter];
-        __syncthreads();  // every wave is done reading s_stage / s_size of the input side
-#pragma unroll
-        for (int it = 0; it < kIter; ++it) {
-            uint32_t size;
-            analyse8(v[it], k, a[it], sb[it], hd[it], size);
-            if (k == 0) {
-                const int blk = it * kBlocksPerIter + quad;
-                s_size[blk] = size;
-                s_hdr[0][blk] = (uint8_t)hd[it];
-            }
-        }
+__global__ __launch_bounds__(1024) void k_in_scan(const uint32_t *__restrict__ totals, uint32_t n_tiles,
+                                                  uint64_t base, uint64_t *__restrict__ ofs)
+{
+    __shared__ uint64_t s_part[1024];
+    const uint32_t per = (n_tiles + 1023u) / 1024u;
+    const uint32_t lo = threadIdx.x * per;
+    const uint32_t hi = lo + per < n_tiles ? lo + per : n_tiles;
+    uint64_t sum = 0;
+    for (uint32_t i = lo; i < hi; ++i) sum += totals[i];
+    s_part[threadIdx.x] = sum;
+    __syncthreads();
+    // Hillis-Steele inclusive scan of the 1024 partial sums
+    for (uint32_t d = 1; d < 1024; d <<= 1) {
+        const uint64_t add = threadIdx.x >= d ? s_part[threadIdx.x - d] : 0;
         __syncthreads();
-        if (tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr[0][tid];
-        uint32_t total = 0;
-        if (wave == 0) total = tile_scan(s_size, s_ofs[0], lane);
+        s_part[threadIdx.x] += add;
         __syncthreads();
-        // ---- wave 0 resolves the global offset while the others pack (HomComp/src/GSZ.cu:170-239)
-        if (wave == 0) {
-            const uint64_t excl = lookback(p.status[kOutChain], tile, p.epoch, total, lane);
-            if (lane == 0) {
-                s_base[0] = p.hdr_bytes + excl;
-                s_total[0] = total;
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < kIter; ++it) {
-            const int blk = it * kBlocksPerIter + quad;
-            pack8(s_stage[0], s_ofs[0][blk], hd[it], k, a[it], sb[it]);
-        }
-        __syncthreads();
-        // ---- coalesced copy of the tile payload to its place in the stream
-        const uint64_t gofs = s_base[0];
-        const uint32_t tot = s_total[0];
-        uint8_t *g = p.out_cmp + gofs;
-        const uint32_t mis = (uint32_t)((uintptr_t)g & 15u);
-        uint32_t head = (16u - mis) & 15u;
-        if (head > tot) head = tot;
-        const uint32_t body = tot - head;
-        const uint32_t nch = body >> 4;
-        const uint32_t tail = body & 15u;
-        if ((uint32_t)tid < head) g[tid] = s_stage[0][tid];
-        const uint32_t *sw = reinterpret_cast<const uint32_t *>(s_stage[0]);
-        for (uint32_t c = tid; c < nch; c += kWG) {
-            const uint32_t s = head + 16u * c;
-            const uint32_t w0 = s >> 2, sh = s & 3u;
-            const uint32_t x0 = sw[w0], x1 = sw[w0 + 1], x2 = sw[w0 + 2], x3 = sw[w0 + 3], x4 = sw[w0 + 4];
-            uint4 o;
-            o.x = __builtin_amdgcn_alignbyte(x1, x0, sh);
-            o.y = __builtin_amdgcn_alignbyte(x2, x1, sh);
-            o.z = __builtin_amdgcn_alignbyte(x3, x2, sh);
-            o.w = __builtin_amdgcn_alignbyte(x4, x3, sh);
-            *reinterpret_cast<uint4 *>(g + s) = o;
-        }
-        if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = s_stage[0][head + 16u * nch + tid];
-        // ---- true stream length = absolute end offset of the last tile (HomComp/src/GSZ.cu:752-755)
-        if (tile == p.n_tiles - 1 && tid == 0) {
-            const uint64_t len = gofs + tot;
-            *p.total = len;
-            if (p.user_total) *p.user_total = len;
-        }
     }
+    uint64_t run = base + s_part[threadIdx.x] - sum;
+    for (uint32_t i = lo; i < hi; ++i) {
+        ofs[i] = run;
+        run += totals[i];
+    }
+    if (threadIdx.x == 1023) ofs[n_tiles] = base + s_part[1023];
 }
 
 // HomComp/src/homcomp.cu:1553-1602: Lorenzo deltas of the quantised values as int32.
@@ -371,17 +498,51 @@ __global__ void k_fill_u64(uint64_t *p, uint64_t n)
 // ---------------------------------------------------------------- launchers
 
 template <int NIN, int LOCAL, int OUT>
-static hipError_t launch_tile(const TileParams &p, hipStream_t s)
+static hipError_t launch_tile(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(p.n_tiles), dim3(kWG), 0, s, p);
+    const uint32_t grid = p.n_tiles < max_grid ? p.n_tiles : max_grid;
+    hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), 0, s, p);
     return hipGetLastError();
 }
 
-hipError_t launch_compress(const TileParams &p, hipStream_t s) { return launch_tile<0, kLocalF32, kOutStream>(p, s); }
-hipError_t launch_decompress(const TileParams &p, hipStream_t s) { return launch_tile<1, kLocalNone, kOutF32>(p, s); }
-hipError_t launch_hom_sum_f32(const TileParams &p, hipStream_t s) { return launch_tile<1, kLocalF32, kOutStream>(p, s); }
-hipError_t launch_hom_sum_i32(const TileParams &p, hipStream_t s) { return launch_tile<1, kLocalI32, kOutStream>(p, s); }
-hipError_t launch_hom_add(const TileParams &p, hipStream_t s) { return launch_tile<2, kLocalNone, kOutStream>(p, s); }
+template <int NIN, int LOCAL, int OUT>
+static hipError_t resident_blocks(int *blocks_per_cu)
+{
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_tile<NIN, LOCAL, OUT>, kWG, 0);
+}
+
+hipError_t tile_kernel_residency(int op, int *blocks_per_cu)
+{
+    switch (op) {
+    case kOpCompress: return resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu);
+    case kOpDecompress: return resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu);
+    case kOpHomSumF32: return resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu);
+    case kOpHomSumI32: return resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu);
+    case kOpHomAdd: return resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
+{
+    switch (op) {
+    case kOpCompress: return launch_tile<0, kLocalF32, kOutStream>(p, max_grid, s);
+    case kOpDecompress: return launch_tile<1, kLocalNone, kOutF32>(p, max_grid, s);
+    case kOpHomSumF32: return launch_tile<1, kLocalF32, kOutStream>(p, max_grid, s);
+    case kOpHomSumI32: return launch_tile<1, kLocalI32, kOutStream>(p, max_grid, s);
+    case kOpHomAdd: return launch_tile<2, kLocalNone, kOutStream>(p, max_grid, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
+                             uint64_t *ofs, hipStream_t s)
+{
+    const uint32_t pieces = n_tiles * 8u;
+    hipLaunchKernelGGL(k_in_totals, dim3((pieces + 255u) / 256u), dim3(256), 0, s, hdr, n_tiles, totals);
+    hipLaunchKernelGGL(k_in_scan, dim3(1), dim3(1024), 0, s, totals, n_tiles, base, ofs);
+    return hipGetLastError();
+}
 
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s)
 {

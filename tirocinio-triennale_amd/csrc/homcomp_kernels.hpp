@@ -8,37 +8,43 @@ namespace hc {
 
 enum : int { kLocalNone = 0, kLocalF32 = 1, kLocalI32 = 2 };   // local operand of the combine stage
 enum : int { kOutStream = 0, kOutF32 = 1 };                    // what a tile produces
-constexpr int kOutChain = 2;                                    // status chain of the output stream
+enum : int { kOpCompress = 0, kOpDecompress, kOpHomSumF32, kOpHomSumI32, kOpHomAdd, kOpCount };
 
 // Geometry shared with the host (must match homcomp_device.hpp).
 constexpr uint32_t kHostTileElems = 4096;
 constexpr uint32_t kHostTileBlocks = 128;
 constexpr uint32_t kHostChunkElems = 32768;
+constexpr uint32_t kHostGroupTiles = 64;
+constexpr uint32_t kHostAccStride = 16;   // 64-bit words between two group accumulators
 
 struct TileParams {
-    const uint8_t *in[2];     // incoming streams (header + payload)
-    uint64_t in_size[2];      // their stated sizes (out-of-bound rule)
-    const void *local;        // float32 values or int32 deltas, n elements, 16-byte aligned
-    uint8_t *out_cmp;         // outgoing stream
-    float *out_f32;           // decompressed values
-    uint64_t n;               // elements
-    uint64_t hdr_bytes;       // header region = one byte per block of the 32768-padded length
-    uint32_t n_tiles;         // padded length / 4096
+    const uint8_t *in[2];       // incoming streams (header + payload)
+    uint64_t in_size[2];        // their stated sizes (out-of-bound rule)
+    const uint64_t *in_ofs[2];  // per stream: absolute payload offset of every tile, n_tiles + 1 entries
+    const void *local;          // float32 values or int32 deltas, n elements, 16-byte aligned
+    uint8_t *out_cmp;           // outgoing stream
+    float *out_f32;             // decompressed values
+    uint64_t n;                 // elements
+    uint64_t hdr_bytes;         // header region = one byte per block of the 32768-padded length
+    uint32_t n_tiles;           // padded length / 4096
     float eb;
-    float recip;              // fl(0.5f / eb), rounded on the host
-    uint64_t *status[3];      // tile status words: incoming 0, incoming 1, outgoing
-    uint32_t *ticket;         // tile index dispenser
-    uint32_t ticket_base;     // dispenser value when this launch starts
-    uint32_t epoch;           // tag that makes this launch's status words distinguishable
-    uint64_t *total;          // receives the stream length
-    uint64_t *user_total;     // optional second destination for the stream length
+    float recip;                // fl(0.5f / eb), rounded on the host
+    uint64_t *tile_status;      // output-offset scan: one word per tile,
+    uint64_t *group_acc;        // one accumulator (zero at launch)
+    uint64_t *group_prefix;     // and one prefix word per group of 64 tiles
+    uint32_t epoch;             // tag that makes this launch's status words distinguishable
+    uint32_t spin_limit;        // bound on unsuccessful scan probes before *error is raised
+    uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
+    uint64_t *total;            // receives the stream length
+    uint64_t *user_total;       // optional second destination for the stream length
 };
 
-hipError_t launch_compress(const TileParams &p, hipStream_t s);
-hipError_t launch_decompress(const TileParams &p, hipStream_t s);
-hipError_t launch_hom_sum_f32(const TileParams &p, hipStream_t s);
-hipError_t launch_hom_sum_i32(const TileParams &p, hipStream_t s);
-hipError_t launch_hom_add(const TileParams &p, hipStream_t s);
+// Resident workgroups per compute unit for one of the tile kernels (sizes the persistent grid).
+hipError_t tile_kernel_residency(int op, int *blocks_per_cu);
+hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
+// Tile payload offsets of an incoming stream from its header bytes.
+hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
+                             uint64_t *ofs, hipStream_t s);
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s);
 hipError_t launch_range(const float *x, uint64_t n, float *partial, uint32_t max_partials,
                         float *out, hipStream_t s);
