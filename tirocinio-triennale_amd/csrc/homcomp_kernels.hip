@@ -110,10 +110,14 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
     if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = stage[head + 16u * nch + tid];
 }
 
+template <int OUT>
+constexpr int tile_threads() { return kWG; }
+
 template <int NIN, int LOCAL, int OUT>
-__global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
+__global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p)
 {
     constexpr bool kEnc = OUT == kOutStream;
+    constexpr int kLead = tile_threads<OUT>() - kWG;
     constexpr int kIn = NIN > 0 ? NIN : 1;
     __shared__ __align__(16) uint8_t s_in[kIn][NIN > 0 ? kStageBytes : 16];
     __shared__ __align__(16) uint8_t s_out[2][kEnc ? kOutStageBytes : 16];
@@ -125,32 +129,39 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
     __shared__ uint64_t s_base;
     __shared__ uint32_t s_total;
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int tid = (int)threadIdx.x - kLead;   // data lane index, negative in the scan wave
+    const bool data = tid >= 0;                 // wave-uniform
+    const bool scanw = threadIdx.x < 64;        // the wave that runs tile-local and global scans
+    const int lane = threadIdx.x & 63;
     const int k = tid & 3;
     const int quad = tid >> 2;
     const int64_t G = gridDim.x;
     const int64_t n_tiles = p.n_tiles;
     const ScanCtx scan{p.tile_status, p.group_acc, p.group_prefix, p.n_tiles, p.epoch, p.spin_limit, p.error};
 
-    LocalRegs<LOCAL> nxt;
-    if ((int64_t)blockIdx.x < n_tiles)
-        load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)blockIdx.x * kTileElems, tid);
+    // The local operand is prefetched two rounds ahead into two register sets that the rounds
+    // use alternately.  A wave's memory operations complete in issue order and s_waitcnt can only
+    // wait for "all but the N youngest", so a load must never be waited for while younger bulk
+    // loads are still in flight: every load here is at least one full round old when it is used.
+    LocalRegs<LOCAL> buf_a, buf_b;
+    if (data && (int64_t)blockIdx.x < n_tiles)
+        load_local<LOCAL>(buf_a, p.local, p.n, (uint64_t)blockIdx.x * kTileElems, tid);
+    if (data && (int64_t)blockIdx.x + G < n_tiles)
+        load_local<LOCAL>(buf_b, p.local, p.n, (uint64_t)(blockIdx.x + G) * kTileElems, tid);
 
     // scan pipeline registers of wave 0: byte totals of the tiles of the previous two rounds and
     // the probe that was issued in the previous round for the older of the two
     uint32_t total1 = 0, total2 = 0;
     ScanProbe probe{0, 0, 0};
 
-    // Round i handles tile t0 = blockIdx.x + i*G and, on the encoder, finishes the scan and the
-    // store of the tiles of the two rounds before (t1, t2).
-    for (int64_t t0 = blockIdx.x;; t0 += G) {
+    // A round handles tile t0 (operand in `nxt`) and, on the encoder, finishes the scan and the
+    // store of the tiles of the two rounds before (t1, t2).  Returns false when nothing is left.
+    auto round = [&](const int64_t t0, LocalRegs<LOCAL> &nxt) __attribute__((always_inline)) -> bool {
         const int64_t t1 = t0 - G, t2 = t0 - 2 * G;
         const bool v0 = t0 < n_tiles;
         const bool v1 = kEnc && t1 >= 0 && t1 < n_tiles;
         const bool v2 = kEnc && t2 >= 0 && t2 < n_tiles;
-        if (!v0 && !v1 && !v2) break;
+        if (!v0 && !v1 && !v2) return false;
         const uint32_t tile = (uint32_t)t0;
         const int buf = (int)((t0 / G) & 1);
 
@@ -166,7 +177,7 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                 const uint64_t start = p.in_ofs[c][tile];
                 const uint32_t total = (uint32_t)(p.in_ofs[c][tile + 1] - start);
                 in_base[c] = start;
-                if (tid < kTileBlocks) {
+                if (data && tid < kTileBlocks) {
                     const uint32_t h = p.in[c][(uint64_t)tile * kTileBlocks + tid];
                     s_hdr_in[c][tid] = (uint8_t)h;
                     s_size[tid] = size_from_header(h);
@@ -176,8 +187,8 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                 const uint32_t shift = (uint32_t)(g0 - ga);
                 in_shift[c] = shift;
                 const uint32_t nbytes = total ? shift + total : 0u;
-                const uint32_t nchunks = (nbytes + 15u) >> 4;
-                for (uint32_t i = tid; i < nchunks; i += kWG) {
+                const uint32_t nchunks = data ? (nbytes + 15u) >> 4 : 0u;
+                for (uint32_t i = (uint32_t)tid; i < nchunks; i += kWG) {
                     if (16u * (i + 1u) <= nbytes) {
                         *reinterpret_cast<u32x4 *>(&s_in[c][16u * i]) =
                             stream_load<u32x4>(reinterpret_cast<const void *>(ga + 16u * (uintptr_t)i));
@@ -187,10 +198,11 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                     }
                 }
                 __syncthreads();
-                if (wave == 0) tile_scan(s_size, s_ofs_in[c], lane);
+                if (scanw) tile_scan(s_size, s_ofs_in[c], lane);
                 __syncthreads();
             }
 
+            if (data) {
             // ---- per iteration: local deltas + decoded deltas
             int32_t v[kIter][8];
 #pragma unroll
@@ -229,11 +241,10 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                 }
             }
 
-            // ---- the local operand of the next round starts to fly now
-            if (t0 + G < n_tiles)
-                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + G) * kTileElems, tid);
-
             if constexpr (!kEnc) {
+                // ---- the operand of the round after the next one starts to fly now
+                if (t0 + 2 * G < n_tiles)
+                    load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
                 // ---- HomComp/src/GSZ.cu:1426-1468: running sum inside the block, dequantise, store
 #pragma unroll
                 for (int it = 0; it < kIter; ++it) {
@@ -259,7 +270,6 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                             if (e0 + m < p.n) p.out_f32[e0 + m] = y[m];
                     }
                 }
-                __syncthreads();  // LDS of this tile is dead before the next round overwrites it
             } else {
                 // ---- rate selection and header bytes (HomComp/src/GSZ.cu:151-167)
 #pragma unroll
@@ -273,20 +283,16 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                     }
                 }
             }
+            }  // data
+            if constexpr (!kEnc) __syncthreads();  // LDS of this tile is dead before the next round overwrites it
         }
 
         if constexpr (kEnc) {
             __syncthreads();
-            if (v0 && tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr_out[tid];
-            // ---- wave 0: tile-local scan and the scan steps (HomComp/src/GSZ.cu:170-239): publish
-            //      this round's tile, resolve the tile of two rounds ago from the probe issued in
-            //      the previous round, issue the probe for the previous round's tile
-            if (wave == 0) {
-                uint32_t total0 = 0;
-                if (v0) {
-                    total0 = tile_scan(s_size, s_ofs_out, lane);
-                    scan_publish(scan, tile, total0, lane);
-                }
+            // ---- wave 0 runs the scan steps (HomComp/src/GSZ.cu:170-239).  Order matters: a wave's
+            //      memory operations complete in issue order, so the resolve step, which waits for
+            //      the probe issued a round ago, comes before this round's stores and loads.
+            if (scanw) {
                 if (v2) {
                     const uint64_t excl = scan_resolve(scan, (uint32_t)t2, total2, probe, lane);
                     if (lane == 0) {
@@ -294,13 +300,23 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                         s_total = total2;
                     }
                 }
+                uint32_t total0 = 0;
+                if (v0) {
+                    total0 = tile_scan(s_size, s_ofs_out, lane);
+                    scan_publish(scan, tile, total0, lane);
+                }
                 if (v1) probe = scan_probe(scan, (uint32_t)t1, lane);
                 total2 = total1;
                 total1 = total0;
             }
             __syncthreads();
+            // ---- the operand of the round after the next one starts to fly now (after the scan
+            //      steps, so that the scan wave never waits behind these loads)
+            if (data && t0 + 2 * G < n_tiles)
+                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
+            if (v0 && data && tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr_out[tid];
             // ---- the tile packed two rounds ago goes to its place in the stream
-            if (v2) {
+            if (v2 && data) {
                 const uint64_t gofs = s_base;
                 const uint32_t tot = s_total;
                 copy_out(s_out[buf], p.out_cmp + gofs, tot, tid);
@@ -313,7 +329,7 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
             }
             __syncthreads();
             // ---- and this round's tile takes over the buffer (HomComp/src/GSZ.cu:241-751)
-            if (v0) {
+            if (v0 && data) {
 #pragma unroll
                 for (int it = 0; it < kIter; ++it) {
                     const int blk = it * kBlocksPerIter + quad;
@@ -321,6 +337,12 @@ __global__ __launch_bounds__(kWG) void k_tile(const TileParams p)
                 }
             }
         }
+        return true;
+    };
+
+    for (int64_t t0 = blockIdx.x;; t0 += 2 * G) {
+        if (!round(t0, buf_a)) break;
+        if (!round(t0 + G, buf_b)) break;
     }
 }
 
@@ -501,14 +523,15 @@ template <int NIN, int LOCAL, int OUT>
 static hipError_t launch_tile(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     const uint32_t grid = p.n_tiles < max_grid ? p.n_tiles : max_grid;
-    hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), 0, s, p);
+    hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(grid), dim3(tile_threads<OUT>()), 0, s, p);
     return hipGetLastError();
 }
 
 template <int NIN, int LOCAL, int OUT>
 static hipError_t resident_blocks(int *blocks_per_cu)
 {
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_tile<NIN, LOCAL, OUT>, kWG, 0);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_tile<NIN, LOCAL, OUT>,
+                                                        tile_threads<OUT>(), 0);
 }
 
 hipError_t tile_kernel_residency(int op, int *blocks_per_cu)
