@@ -385,12 +385,22 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
 __global__ __launch_bounds__(1024) void k_in_scan(const uint32_t *__restrict__ totals, uint32_t n_tiles,
                                                   uint64_t base, uint64_t *__restrict__ ofs)
 {
+    // Each thread owns a contiguous run of `per` tiles (a multiple of 4, read as 16-byte
+    // vectors with all loads of a pass in flight together); n_tiles is a multiple of 8.
     __shared__ uint64_t s_part[1024];
-    const uint32_t per = (n_tiles + 1023u) / 1024u;
+    constexpr uint32_t kVec = 4, kUnroll = 4;
+    const uint32_t per = (((n_tiles + 1023u) / 1024u) + kVec - 1u) / kVec * kVec;
     const uint32_t lo = threadIdx.x * per;
-    const uint32_t hi = lo + per < n_tiles ? lo + per : n_tiles;
+    const uint32_t hi = lo + per < n_tiles ? lo + per : n_tiles;   // lo, hi multiples of 4 (or lo >= hi)
     uint64_t sum = 0;
-    for (uint32_t i = lo; i < hi; ++i) sum += totals[i];
+    for (uint32_t i = lo; i < hi; i += kVec * kUnroll) {
+        u32x4 q[kUnroll];
+#pragma unroll
+        for (uint32_t u = 0; u < kUnroll; ++u)
+            q[u] = i + u * kVec < hi ? *reinterpret_cast<const u32x4 *>(totals + i + u * kVec) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (uint32_t u = 0; u < kUnroll; ++u) sum += (uint64_t)q[u].x + q[u].y + q[u].z + q[u].w;
+    }
     s_part[threadIdx.x] = sum;
     __syncthreads();
     // Hillis-Steele inclusive scan of the 1024 partial sums
@@ -401,9 +411,16 @@ __global__ __launch_bounds__(1024) void k_in_scan(const uint32_t *__restrict__ t
         __syncthreads();
     }
     uint64_t run = base + s_part[threadIdx.x] - sum;
-    for (uint32_t i = lo; i < hi; ++i) {
-        ofs[i] = run;
-        run += totals[i];
+    for (uint32_t i = lo; i < hi; i += kVec) {
+        const u32x4 q = *reinterpret_cast<const u32x4 *>(totals + i);
+        uint64_t o[4];
+        o[0] = run;
+        o[1] = o[0] + q.x;
+        o[2] = o[1] + q.y;
+        o[3] = o[2] + q.z;
+        run = o[3] + q.w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ofs[i + j] = o[j];
     }
     if (threadIdx.x == 1023) ofs[n_tiles] = base + s_part[1023];
 }
