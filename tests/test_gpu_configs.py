@@ -1,0 +1,119 @@
+"""The named benchmark configurations at their full sizes, on the GPU, against the CPU oracle
+(run with OpenMP) on the very same buffers:
+
+  config 2  64M float32 smooth, REL eb 1e-4 and 1e-3: one compress + one decompress
+  config 3  256M float32 (1 GiB) gradient-like, ABS eb 1e-6: wide bit widths, outliers
+  config 4  ring reduce-scatter on one GPU: 8 rank buffers x 32M floats in 8 chunks, 8 compresses
+            + 56 homomorphic sums in 7 sequential waves (the schedule of
+            HomComp/src/cuda_awareallreduce.cu:205-235 with the MPI exchange left out)
+
+Streams are compared byte for byte, decompressed values bit for bit, the ring result against
+integer addition of the ranks' quantised values.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_compress(pkg, ws, torch, x, eb):
+    cmp = torch.empty(pkg.max_stream_bytes(x.numel()), dtype=torch.uint8, device="cuda")
+    ws.compress(x, float(eb), cmp)
+    return cmp, ws.last_size()
+
+
+def check_roundtrip(pkg, orc, torch, x, eb, n_way=1):
+    n = x.numel()
+    with pkg.Workspace(n) as ws:
+        cmp, L = gpu_compress(pkg, ws, torch, x, eb)
+        dec = torch.empty(n, dtype=torch.float32, device="cuda")
+        ws.decompress(cmp, L, n, float(eb), dec)
+        torch.cuda.synchronize()
+        xh = x.cpu().numpy()
+        want = orc.compress(xh, eb)
+        got = cmp[:L].cpu().numpy()
+        assert L == want.size and np.array_equal(got, want), "stream differs from the oracle"
+        want_dec = orc.decompress(want, n, eb)
+        got_dec = dec.cpu().numpy()
+        assert np.array_equal(got_dec.view(np.uint32), want_dec.view(np.uint32))
+        err = np.abs(got_dec.astype(np.float64) - xh.astype(np.float64))
+        assert (err <= float(eb) + 2.0 ** -21 * np.abs(xh)).all()
+        # size-independent property: recompressing the reconstruction reproduces the stream
+        cmp2, L2 = gpu_compress(pkg, ws, torch, dec, eb)
+        assert L2 == L and torch.equal(cmp2[:L2], cmp[:L])
+        return 4.0 * n / L
+
+
+@pytest.mark.parametrize("rel", [1e-4, 1e-3])
+def test_config2_smooth_64m(pkg, orc, gen, cuda, rel):
+    orc.set_threads(16)
+    n = 1 << 26
+    x = gen.smooth_torch(n, seed=1)
+    mm = cuda.empty(2, dtype=cuda.float32, device="cuda")
+    with pkg.Workspace(n) as ws:
+        ws.value_range(x, mm)
+    mn, mx = mm.cpu().numpy()
+    eb = np.float32(pkg.rel_to_abs(rel, float(mn), float(mx)))
+    xh_mn, xh_mx = orc.value_range(x.cpu().numpy())
+    assert (mn, mx) == (xh_mn, xh_mx) and eb == orc.rel_to_abs(rel, xh_mn, xh_mx)
+    cr = check_roundtrip(pkg, orc, cuda, x, eb)
+    assert cr > 5.0
+
+
+def test_config3_gradient_like_1gib(pkg, orc, gen, cuda):
+    orc.set_threads(16)
+    n = 1 << 28
+    x = gen.gradient_like_torch(n, seed=1)
+    cr = check_roundtrip(pkg, orc, cuda, x, np.float32(1e-6))
+    assert 2.0 < cr < 3.5
+
+
+def test_config4_ring_reduce_scatter(pkg, orc, gen, cuda):
+    torch = cuda
+    orc.set_threads(16)
+    ranks, n_rank = 8, 1 << 25
+    chunk = n_rank // ranks
+    data = [gen.smooth_torch(n_rank, seed=10 + r) for r in range(ranks)]
+    # one absolute bound shared by all ranks: REL 1e-4 of the union range
+    mm = torch.empty(2 * ranks, dtype=torch.float32, device="cuda")
+    with pkg.Workspace(n_rank) as ws:
+        for r in range(ranks):
+            ws.value_range(data[r], mm[2 * r:2 * r + 2])
+    m = mm.cpu().numpy()
+    eb = np.float32(pkg.rel_to_abs(1e-4, float(m[0::2].min()), float(m[1::2].max())))
+    cap = pkg.max_stream_bytes(chunk)
+    cur = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    nxt = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    sizes = [0] * ranks
+    with pkg.Workspace(chunk) as ws:
+        # step 0: rank r compresses its own chunk r
+        for r in range(ranks):
+            ws.compress(data[r][r * chunk:(r + 1) * chunk], float(eb), cur[r])
+            sizes[r] = ws.last_size()
+        # steps 1..7: the stream of chunk r moves on to rank (r + k) and takes in its copy of chunk r
+        for k in range(1, ranks):
+            for r in range(ranks):
+                owner = (r + k) % ranks
+                ws.hom_sum_f32(cur[r], sizes[r], data[owner][r * chunk:(r + 1) * chunk], float(eb), nxt[r])
+                sizes[r] = ws.last_size()
+            cur, nxt = nxt, cur
+        torch.cuda.synchronize()
+    host = [d.cpu().numpy() for d in data]
+    for r in range(ranks):
+        sl = slice(r * chunk, (r + 1) * chunk)
+        q_sum = np.zeros(chunk, np.int64)
+        for h in host:
+            q_sum += orc.quantize_array(h[sl], eb)
+        stream = cur[r][:sizes[r]].cpu().numpy()
+        assert np.array_equal(orc.decode_quants(stream, chunk).astype(np.int64), q_sum), f"chunk {r}"
+        # the GPU stream equals the oracle's chain of the same 7 steps
+        ref = orc.compress(host[r][sl], eb)
+        for k in range(1, ranks):
+            ref = orc.hom_sum_f32(ref, host[(r + k) % ranks][sl], eb)
+        assert stream.size == ref.size and np.array_equal(stream, ref), f"chunk {r} stream"
+        # error of the reduced chunk: at most 8 * eb (+ float32 slack)
+        dec = orc.decompress(stream, chunk, eb).astype(np.float64)
+        exact = np.zeros(chunk, np.float64)
+        for h in host:
+            exact += h[sl]
+        assert (np.abs(dec - exact) <= ranks * float(eb) * (1 + 1e-3)).all()

@@ -1,0 +1,126 @@
+// Drop-in for the reference's host API (HomComp/include/GSZ_entry.h:14-37 and the directly
+// launched kernel of HomComp/include/homcomp.cuh:2-5) on top of the C ABI of include/homcomp.h.
+//
+// Same names, argument order and meaning as the reference, with cudaStream_t -> hipStream_t:
+//   * errorBound is an absolute bound;
+//   * every call is synchronous with respect to the host, as in the reference (its wrappers
+//     end in a blocking cudaMemcpy / cudaFree): the size is read back before returning;
+//   * *cmpSize receives what the reference's wrappers report, L + nbEle_padded/32
+//     (HomComp/src/GSZ_entry.cu:291-295 adds the header length a second time); define
+//     HOMCOMP_TRUE_CMPSIZE to receive the true stream length L instead;
+//   * like the reference, the functions return void; failures are reported through
+//     homcomp::last_status() (0 = ok), which a caller can poll where the reference polls
+//     cudaGetLastError() (HomComp/src/cuda_awareallreduce.cu:207).
+// The scratch arrays the reference allocates and frees on every call live in a per-thread
+// workspace that grows on demand.  d_cmpBytes needs homcomp_max_stream_bytes(nbEle) bytes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+
+#include "../../include/homcomp.h"
+
+namespace homcomp {
+
+inline int &last_status()
+{
+    thread_local int status = HOMCOMP_OK;
+    return status;
+}
+
+namespace detail {
+
+struct Cache {
+    homcomp_workspace *ws = nullptr;
+    size_t capacity = 0;
+    ~Cache() { if (ws) homcomp_workspace_destroy(ws); }
+};
+
+inline homcomp_workspace *workspace(size_t nbEle)
+{
+    thread_local Cache cache;
+    if (!cache.ws || cache.capacity < nbEle) {
+        if (cache.ws) homcomp_workspace_destroy(cache.ws);
+        cache.ws = nullptr;
+        cache.capacity = 0;
+        const int rc = homcomp_workspace_create(&cache.ws, nbEle);
+        if (rc != HOMCOMP_OK) {
+            last_status() = rc;
+            return nullptr;
+        }
+        cache.capacity = nbEle;
+    }
+    return cache.ws;
+}
+
+inline void report_size(homcomp_workspace *ws, int rc, size_t nbEle, size_t *cmpSize, hipStream_t stream)
+{
+    size_t len = 0;
+    if (rc == HOMCOMP_OK) rc = homcomp_last_size(ws, &len, stream);
+    last_status() = rc;
+#ifdef HOMCOMP_TRUE_CMPSIZE
+    *cmpSize = len;
+    (void)nbEle;
+#else
+    *cmpSize = homcomp_ref_cmpsize(len, nbEle);
+#endif
+}
+
+}  // namespace detail
+}  // namespace homcomp
+
+// HomComp/include/GSZ_entry.h:14-16
+inline void GSZ_compress_deviceptr_outlier(float *d_oriData, unsigned char *d_cmpBytes, size_t nbEle,
+                                           size_t *cmpSize, float errorBound, hipStream_t stream = 0)
+{
+    homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
+    if (!ws) return;
+    const int rc = homcomp_compress_f32(ws, d_oriData, nbEle, errorBound, d_cmpBytes, nullptr, stream);
+    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+}
+
+// HomComp/include/GSZ_entry.h:17-20.  cmpSize may be either convention: blocks are only skipped
+// when their payload starts at or beyond it (HomComp/src/GSZ.cu:908-911).
+inline void GSZ_decompress_deviceptr_outlier(float *d_decData, unsigned char *d_cmpBytes, size_t nbEle,
+                                             size_t cmpSize, float errorBound, hipStream_t stream = 0)
+{
+    homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
+    if (!ws) return;
+    int rc = homcomp_decompress_f32(ws, d_cmpBytes, cmpSize, nbEle, errorBound, d_decData, stream);
+    if (rc == HOMCOMP_OK && hipStreamSynchronize(stream) != hipSuccess) rc = HOMCOMP_ERR_HIP;
+    homcomp::last_status() = rc;
+}
+
+// HomComp/include/GSZ_entry.h:29-32
+inline void homomorphic_sum(unsigned char *d_cmpBytesIn, int *d_quantPredLoc, unsigned char *d_cmpByteOut,
+                            size_t nbEle, float errorBound, size_t *cmpSize, size_t cmpSizeCmpBlock,
+                            hipStream_t stream = 0)
+{
+    (void)errorBound;  // the integer path does not quantise
+    homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
+    if (!ws) return;
+    const int rc = homcomp_hom_sum_i32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_quantPredLoc, nbEle,
+                                       d_cmpByteOut, nullptr, stream);
+    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+}
+
+// HomComp/include/GSZ_entry.h:33-36
+inline void homomorphic_sum_F(unsigned char *d_cmpBytesIn, float *d_localChunk, unsigned char *d_cmpByteOut,
+                              size_t nbEle, float errorBound, size_t *cmpSize, size_t cmpSizeCmpBlock,
+                              hipStream_t stream = 0)
+{
+    homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
+    if (!ws) return;
+    const int rc = homcomp_hom_sum_f32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_localChunk, nbEle, errorBound,
+                                       d_cmpByteOut, nullptr, stream);
+    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+}
+
+// Callers of the reference launch kernel_quant_prediction<<<grid, 32, 0, stream>>>(...) directly
+// (HomComp/src/cuda_awareallreduce.cu:103); this is the same operation as a function.
+inline void kernel_quant_prediction(const float *d_localData, int *d_quantPredData, float errorBound,
+                                    size_t nbEle, hipStream_t stream = 0)
+{
+    homcomp::last_status() = homcomp_quant_predict_f32(d_localData, nbEle, errorBound, d_quantPredData, stream);
+}
