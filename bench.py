@@ -78,6 +78,8 @@ def main() -> int:
     ap.add_argument("--abs", type=float, default=None, help="absolute error bound (overrides --rel)")
     ap.add_argument("--cpu-sample-log2", type=int, default=24)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1:1 copy of an operand (reference point for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; --gpus above 1 is not part of this build "
@@ -146,6 +148,12 @@ def main() -> int:
     add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n)
     add("hom_add", lambda: ws.hom_add(cmp_a, la, cmp_b, lb, n, cmp_s), la + lb + ls)
     torch.cuda.synchronize()
+    if args.copy_calibration:
+        # a copy kernel of known size: reads 4N bytes and writes 4N bytes
+        ms = time_op(torch, lambda: dec.copy_(x), 3)
+        ops["copy_calibration"] = {"ms": round(ms, 4), "alg_bytes": 8 * n,
+                                   "achieved_GBps": round(8 * n / ms / 1e6, 1),
+                                   "frac_hbm": round(8 * n / (ms * 1e-3) / HBM_PEAK, 4)}
 
     dom = "hom_sum_f32"
     roofline = {"bound": "hbm", "kernel": dom, "achieved": ops[dom]["achieved_GBps"],

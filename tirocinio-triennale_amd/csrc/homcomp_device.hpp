@@ -66,25 +66,34 @@ __device__ __forceinline__ uint32_t quad_or(uint32_t v)
     return v;
 }
 
+constexpr int kDppRowHalfMirror = 0x141;  // lane i reads lane 7-i inside its group of 8
+constexpr int kDppRowMirror = 0x140;      // lane i reads lane 15-i inside its row of 16
+
+// Inclusive scan across the wave: Hillis-Steele with DPP row shifts inside each row of 16 lanes,
+// then the totals of the earlier rows through scalar registers.
 __device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int lane)
 {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        uint32_t t = __shfl_up(x, d, 64);
-        if (lane >= d) x += t;
-    }
-    return x;
+    x += dpp_u32<0x111>(x);   // row_shr:1
+    x += dpp_u32<0x112>(x);   // row_shr:2
+    x += dpp_u32<0x114>(x);   // row_shr:4
+    x += dpp_u32<0x118>(x);   // row_shr:8
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)x, 15);
+    const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)x, 31);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)x, 47);
+    const int row = lane >> 4;
+    return x + (row > 0 ? r0 : 0u) + (row > 1 ? r1 : 0u) + (row > 2 ? r2 : 0u);
 }
 
-__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t x)
+// Sum across the wave (uniform result): DPP butterflies inside each row of 16 lanes, then the four
+// row sums through scalar registers.
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x)
 {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        uint32_t lo = __shfl_xor((uint32_t)x, d, 64);
-        uint32_t hi = __shfl_xor((uint32_t)(x >> 32), d, 64);
-        x += ((uint64_t)hi << 32) | lo;
-    }
-    return x;
+    x += dpp_u32<kDppXor1>(x);
+    x += dpp_u32<kDppXor2>(x);
+    x += dpp_u32<kDppRowHalfMirror>(x);
+    x += dpp_u32<kDppRowMirror>(x);
+    return (uint32_t)__builtin_amdgcn_readlane((int)x, 0) + (uint32_t)__builtin_amdgcn_readlane((int)x, 16) +
+           (uint32_t)__builtin_amdgcn_readlane((int)x, 32) + (uint32_t)__builtin_amdgcn_readlane((int)x, 48);
 }
 
 // ---------------------------------------------------------------- scalar arithmetic
@@ -395,7 +404,8 @@ __device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile
         if (scan_give_up(c, spins, lane)) break;
         pr.wt = scan_probe_tiles(c, tile, lane);
     }
-    uint64_t excl = wave_sum_u64((uint32_t)lane < r ? (pr.wt & kValueMask) : 0ull);
+    // a tile total is below 2^15 and a group accumulator below 2^21, so 32-bit sums are exact
+    uint64_t excl = wave_sum_u32((uint32_t)lane < r ? (uint32_t)pr.wt : 0u);
     // earlier groups: back to the nearest published prefix
     int64_t first = (int64_t)g - 1;
     for (;;) {
@@ -411,11 +421,16 @@ __device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile
             scan_probe_groups(c, first, lane, pr.wa, pr.wp);
             continue;
         }
-        uint64_t v = 0;
-        if (lane < stop) v = pr.wa & 0xffffffffull;
-        else if (lane == stop && gi >= 0) v = pr.wp & kValueMask;
-        excl += wave_sum_u64(v);
-        if (m_prefix) break;
+        excl += wave_sum_u32(lane < stop ? (uint32_t)pr.wa : 0u);
+        if (m_prefix) {
+            // the 40-bit prefix of the stopping group, read from its lane (none before group 0)
+            if (first - stop >= 0) {
+                const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)pr.wp, stop);
+                const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(pr.wp >> 32), stop);
+                excl += (((uint64_t)hi << 32) | lo) & kValueMask;
+            }
+            break;
+        }
         first -= 64;
         scan_probe_groups(c, first, lane, pr.wa, pr.wp);
     }

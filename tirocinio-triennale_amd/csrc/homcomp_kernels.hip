@@ -288,18 +288,18 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
         }
 
         if constexpr (kEnc) {
-            __syncthreads();
-            // ---- wave 0 runs the scan steps (HomComp/src/GSZ.cu:170-239).  Order matters: a wave's
-            //      memory operations complete in issue order, so the resolve step, which waits for
-            //      the probe issued a round ago, comes before this round's stores and loads.
-            if (scanw) {
-                if (v2) {
-                    const uint64_t excl = scan_resolve(scan, (uint32_t)t2, total2, probe, lane);
-                    if (lane == 0) {
-                        s_base = p.hdr_bytes + excl;
-                        s_total = total2;
-                    }
+            // ---- wave 0 runs the scan steps (HomComp/src/GSZ.cu:170-239).  A wave's memory
+            //      operations complete in issue order, so the resolve step, which needs the probe
+            //      issued a round ago, comes before this round's stores and loads of the wave.
+            if (scanw && v2) {
+                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, total2, probe, lane);
+                if (lane == 0) {
+                    s_base = p.hdr_bytes + excl;
+                    s_total = total2;
                 }
+            }
+            __syncthreads();
+            if (scanw) {
                 uint32_t total0 = 0;
                 if (v0) {
                     total0 = tile_scan(s_size, s_ofs_out, lane);
@@ -309,11 +309,6 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
                 total2 = total1;
                 total1 = total0;
             }
-            __syncthreads();
-            // ---- the operand of the round after the next one starts to fly now (after the scan
-            //      steps, so that the scan wave never waits behind these loads)
-            if (data && t0 + 2 * G < n_tiles)
-                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
             if (v0 && data && tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr_out[tid];
             // ---- the tile packed two rounds ago goes to its place in the stream
             if (v2 && data) {
@@ -328,6 +323,9 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
                 }
             }
             __syncthreads();
+            // ---- the operand of the round after the next one starts to fly now
+            if (data && t0 + 2 * G < n_tiles)
+                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
             // ---- and this round's tile takes over the buffer (HomComp/src/GSZ.cu:241-751)
             if (v0 && data) {
 #pragma unroll
