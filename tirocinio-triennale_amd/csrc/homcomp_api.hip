@@ -36,11 +36,9 @@ struct homcomp_workspace {
     int device;
     size_t max_n;
     uint32_t max_tiles;
-    uint32_t max_groups;
     void *d_block;            // one allocation holding everything below
-    uint64_t *d_tile_status;  // [max_tiles]   output-offset scan, tile words
-    uint64_t *d_group_prefix; // [max_groups]  output-offset scan, group prefix words
-    uint64_t *d_group_acc;    // [max_groups * kHostAccStride]  output-offset scan, group accumulators
+    uint64_t *d_tile_totals;   // [max_tiles]  output-offset scan: tile totals
+    uint64_t *d_tile_prefixes; // [max_tiles]  output-offset scan: tile prefixes (adjacent to the totals)
     uint64_t *d_in_ofs[2];    // [max_tiles+1] tile payload offsets of the incoming streams
     uint32_t *d_in_totals;    // [max_tiles]   scratch of the offsets pre-pass
     uint64_t *d_total;        // stream length of the last stream-producing call
@@ -63,12 +61,12 @@ int check_ws(const homcomp_workspace *ws, size_t n)
     return HOMCOMP_OK;
 }
 
-// Fresh epoch for one launch; clears the status words when the 22-bit tag wraps (the two
-// status arrays are adjacent).
+// Fresh epoch for one launch; clears the scan words when the 22-bit tag wraps (the two arrays
+// are adjacent).
 int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
 {
     if (ws->epoch >= kMaxEpoch) {
-        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_status, (uint64_t)ws->max_tiles + ws->max_groups, s)))
+        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)))
             return HOMCOMP_ERR_HIP;
         ws->epoch = 0;
     }
@@ -82,9 +80,8 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
     p->n = n;
     p->hdr_bytes = homcomp_header_bytes(n);
     p->n_tiles = (uint32_t)(padded_len(n) / hc::kHostTileElems);
-    p->tile_status = ws->d_tile_status;
-    p->group_prefix = ws->d_group_prefix;
-    p->group_acc = ws->d_group_acc;
+    p->tile_totals = ws->d_tile_totals;
+    p->tile_prefixes = ws->d_tile_prefixes;
     p->spin_limit = kSpinLimit;
     p->error = ws->d_error;
     p->total = ws->d_total;
@@ -102,11 +99,6 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 
 int run_tile_op(homcomp_workspace *ws, int op, const hc::TileParams &p, hipStream_t s)
 {
-    if (op != hc::kOpDecompress) {
-        // the group accumulators of the output-offset scan start every call at zero
-        const uint64_t groups = (p.n_tiles + hc::kHostGroupTiles - 1) / hc::kHostGroupTiles;
-        if (!hip_ok(hc::launch_fill_u64(ws->d_group_acc, groups * hc::kHostAccStride, s))) return HOMCOMP_ERR_HIP;
-    }
     return hip_ok(hc::launch_tile_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -175,12 +167,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
-    ws->max_groups = (ws->max_tiles + hc::kHostGroupTiles - 1) / hc::kHostGroupTiles;
-    const size_t t = ws->max_tiles, g = ws->max_groups;
+    const size_t t = ws->max_tiles;
     size_t off = 0;
     auto take = [&off](size_t bytes) { size_t o = off; off = (off + bytes + 255) & ~(size_t)255; return o; };
-    const size_t o_status = take((t + g) * sizeof(uint64_t));
-    const size_t o_acc = take(g * hc::kHostAccStride * sizeof(uint64_t));
+    const size_t o_status = take(2 * t * sizeof(uint64_t));
     const size_t o_in0 = take((t + 1) * sizeof(uint64_t));
     const size_t o_in1 = take((t + 1) * sizeof(uint64_t));
     const size_t o_tot = take(t * sizeof(uint32_t));
@@ -194,6 +184,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         ok = hip_ok(hc::tile_kernel_residency(op, &per_cu));
         if (ok && per_cu < 1) per_cu = 1;
         ws->max_grid[op] = (uint32_t)per_cu * (uint32_t)prop.multiProcessorCount;
+        if (ws->max_grid[op] < 2) ws->max_grid[op] = 2;   // an encoder needs a data workgroup and the scan server
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
         !hip_ok(hipHostMalloc((void **)&ws->h_total, 2 * sizeof(uint64_t), hipHostMallocDefault))) {
@@ -202,9 +193,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         return HOMCOMP_ERR_HIP;
     }
     uint8_t *base = (uint8_t *)ws->d_block;
-    ws->d_tile_status = (uint64_t *)(base + o_status);
-    ws->d_group_prefix = ws->d_tile_status + t;
-    ws->d_group_acc = (uint64_t *)(base + o_acc);
+    ws->d_tile_totals = (uint64_t *)(base + o_status);
+    ws->d_tile_prefixes = ws->d_tile_totals + t;
     ws->d_in_ofs[0] = (uint64_t *)(base + o_in0);
     ws->d_in_ofs[1] = (uint64_t *)(base + o_in1);
     ws->d_in_totals = (uint32_t *)(base + o_tot);

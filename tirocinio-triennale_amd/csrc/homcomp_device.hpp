@@ -71,6 +71,8 @@ constexpr int kDppRowMirror = 0x140;      // lane i reads lane 15-i inside its r
 
 // Inclusive scan across the wave: Hillis-Steele with DPP row shifts inside each row of 16 lanes,
 // then the totals of the earlier rows through scalar registers.
+// Inclusive scan across the wave: Hillis-Steele with DPP row shifts inside each row of 16 lanes,
+// then the totals of the earlier rows through scalar registers.
 __device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int lane)
 {
     x += dpp_u32<0x111>(x);   // row_shr:1
@@ -82,18 +84,6 @@ __device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int lane)
     const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)x, 47);
     const int row = lane >> 4;
     return x + (row > 0 ? r0 : 0u) + (row > 1 ? r1 : 0u) + (row > 2 ? r2 : 0u);
-}
-
-// Sum across the wave (uniform result): DPP butterflies inside each row of 16 lanes, then the four
-// row sums through scalar registers.
-__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x)
-{
-    x += dpp_u32<kDppXor1>(x);
-    x += dpp_u32<kDppXor2>(x);
-    x += dpp_u32<kDppRowHalfMirror>(x);
-    x += dpp_u32<kDppRowMirror>(x);
-    return (uint32_t)__builtin_amdgcn_readlane((int)x, 0) + (uint32_t)__builtin_amdgcn_readlane((int)x, 16) +
-           (uint32_t)__builtin_amdgcn_readlane((int)x, 32) + (uint32_t)__builtin_amdgcn_readlane((int)x, 48);
 }
 
 // ---------------------------------------------------------------- scalar arithmetic
@@ -274,41 +264,33 @@ __device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uin
 // ---------------------------------------------------------------- output-offset scan
 //
 // The byte offset of a tile's payload in the outgoing stream is an exclusive prefix sum over
-// all earlier tiles (HomComp/src/GSZ.cu:170-239).  It is resolved in a single pass, without any
-// workgroup ever having to wait for another one in the steady state:
+// all earlier tiles (HomComp/src/GSZ.cu:170-239).  It is resolved in a single pass by a division
+// of labour between the data workgroups and one scan-server workgroup of the same launch:
 //
-//   publish   (round i)    the tile stores its byte total in its tile word and adds it, together
-//                          with a count of one, to the accumulator word of its group of 64 tiles
-//                          (a fire-and-forget atomic);
-//   probe     (round i+1)  the tile's wave issues the loads of: the tile words of the earlier
-//                          tiles of its group, and for the 64 groups before its own the
-//                          accumulator word and the prefix word;
-//   resolve   (round i+2)  the loaded words are a round old and were published two rounds ago:
-//                          exclusive prefix = (nearest published group prefix) + (accumulators of
-//                          the complete groups after it) + (tile words of the group's earlier
-//                          tiles).  The last tile of a group publishes the group's prefix word.
+//   data workgroup, round i     publishes the tile's byte total in the tile's total word
+//   scan server                 sweeps the total words in tile order, 1024 tiles per step, waits
+//                               until they are all there, scans them and writes every tile's
+//                               exclusive prefix into the tile's prefix word
+//   data workgroup, round i+1   issues the load of the prefix word
+//   data workgroup, round i+2   uses it: the payload goes to its place in the stream
 //
-// Tile and prefix words carry an epoch tag: bits 63-62 state (0 empty, 1 tile total, 2 inclusive
-// group prefix), bits 61-40 the call's epoch, bits 39-0 a byte count; a word of another epoch
-// reads as empty, so these arrays are never cleared between calls (the host clears them when the
-// 22-bit epoch wraps).  Accumulator words (bits 39-32 count, bits 31-0 byte sum) are zeroed
-// before every call.
+// so a data workgroup never waits for another data workgroup, only the server waits, and every
+// word is written by one workgroup and read by one.  (Measured on MI355X: read-modify-write
+// atomics on one 128-byte line are serialised at about 11 ns each, and plain loads of a line
+// that is being updated atomically by other compute units are about as slow -- a ticket
+// counter or shared accumulators that thousands of workgroups touch cost more than the codec.)
 //
-// All tiles with a smaller index are processed by workgroups that are resident at the same time
-// (the grid is sized to fit the device), so a missing word is always on its way; if a probe does
-// come back incomplete the wave re-reads until it is complete.  As a guard against a launch that
-// could not become fully resident these waits are bounded: after `spin_limit` unsuccessful
-// re-reads the wave raises *err and goes on with what it has, so the kernel always terminates.
+// A word carries an epoch tag: bits 63-62 state (0 empty, 1 total, 2 exclusive prefix), bits
+// 61-40 the call's epoch, bits 39-0 a byte count; a word of another epoch reads as empty, so the
+// arrays are never cleared between calls (the host clears them when the 22-bit epoch wraps).
+//
+// All workgroups of the launch are resident at the same time (the grid is sized to fit the
+// device), so every word waited for is on its way.  As a guard against a launch that could not
+// become fully resident the waits are bounded: after `spin_limit` unsuccessful re-reads a wave
+// raises *err and goes on with what it has, so the kernel always terminates.
 
 constexpr uint64_t kValueMask = (1ull << 40) - 1;
 constexpr uint32_t kEpochMask = (1u << 22) - 1;
-constexpr int kGroupShift = 6;   // 64 tiles per group
-constexpr uint32_t kGroupMask = (1u << kGroupShift) - 1u;
-constexpr uint32_t kGroupFull = 1u << kGroupShift;
-// Read-modify-write atomics that hit one cache line are serialised by the memory side (about
-// 11 ns each on MI355X, measured), whichever word of the line they address; the accumulators of
-// the groups in flight are updated at the same time, so each gets a 128-byte line of its own.
-constexpr int kAccStride = 16;   // 64-bit words between two accumulators
 
 __device__ __forceinline__ uint64_t status_word(uint32_t epoch, uint32_t state, uint64_t value)
 {
@@ -332,111 +314,45 @@ __device__ __forceinline__ uint32_t status_state(uint64_t w, uint32_t epoch)
 }
 
 struct ScanCtx {
-    uint64_t *tstat;   // tile words
-    uint64_t *gacc;    // group accumulators (zero when the call starts), kAccStride words apart
-    uint64_t *gpref;   // group prefix words
+    uint64_t *totals;     // tile total words, written by the data workgroups
+    uint64_t *prefixes;   // tile prefix words, written by the scan server
     uint32_t n_tiles;
     uint32_t epoch;
     uint32_t spin_limit;
     uint32_t *err;
 };
 
-struct ScanProbe {
-    uint64_t wt;   // lane l: tile word of the l-th tile of the group (l < position in group)
-    uint64_t wa;   // lane l: accumulator of group (first - l)
-    uint64_t wp;   // lane l: prefix word of group (first - l)
-};
-
-__device__ __forceinline__ void scan_publish(const ScanCtx &c, uint32_t tile, uint32_t total, int lane)
-{
-    if (lane == 0) {
-        status_store(&c.tstat[tile], status_word(c.epoch, 1, total));
-        (void)__hip_atomic_fetch_add(&c.gacc[(uint64_t)(tile >> kGroupShift) * kAccStride],
-                                     (1ull << 32) | (uint64_t)total,
-                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-}
-
-__device__ __forceinline__ uint64_t scan_probe_tiles(const ScanCtx &c, uint32_t tile, int lane)
-{
-    return (uint32_t)lane < (tile & kGroupMask) ? status_load(&c.tstat[(tile & ~kGroupMask) + lane]) : 0ull;
-}
-
-__device__ __forceinline__ void scan_probe_groups(const ScanCtx &c, int64_t first, int lane,
-                                                  uint64_t &wa, uint64_t &wp)
-{
-    const int64_t gi = first - lane;
-    wa = 0;
-    wp = 0;
-    if (gi >= 0) {
-        wa = status_load(&c.gacc[gi * kAccStride]);
-        wp = status_load(&c.gpref[gi]);
-    }
-}
-
-__device__ __forceinline__ ScanProbe scan_probe(const ScanCtx &c, uint32_t tile, int lane)
-{
-    ScanProbe pr;
-    pr.wt = scan_probe_tiles(c, tile, lane);
-    scan_probe_groups(c, (int64_t)(tile >> kGroupShift) - 1, lane, pr.wa, pr.wp);
-    return pr;
-}
-
-__device__ __forceinline__ bool scan_give_up(const ScanCtx &c, uint32_t &spins, int lane)
+__device__ __forceinline__ bool scan_give_up(const ScanCtx &c, uint32_t &spins)
 {
     if (++spins > c.spin_limit) {
-        if (lane == 0) atomicOr(c.err, 1u);
+        atomicOr(c.err, 1u);
         return true;
     }
     __builtin_amdgcn_s_sleep(1);
     return false;
 }
 
-// Exclusive prefix of `tile` from an earlier scan_probe(tile); run by one full wave.
-__device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint32_t total,
-                                                 ScanProbe pr, int lane)
+// data side ---------------------------------------------------------------------------------
+
+__device__ __forceinline__ void scan_publish(const ScanCtx &c, uint32_t tile, uint32_t total)
 {
-    const uint32_t g = tile >> kGroupShift;
-    const uint32_t r = tile & kGroupMask;
+    status_store(&c.totals[tile], status_word(c.epoch, 1, total));
+}
+
+__device__ __forceinline__ uint64_t scan_probe(const ScanCtx &c, uint32_t tile)
+{
+    return status_load(&c.prefixes[tile]);
+}
+
+// Exclusive prefix of `tile` from an earlier scan_probe(tile).
+__device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint64_t w)
+{
     uint32_t spins = 0;
-    // earlier tiles of the same group
-    while (__ballot((uint32_t)lane < r && status_state(pr.wt, c.epoch) == 0) != 0) {
-        if (scan_give_up(c, spins, lane)) break;
-        pr.wt = scan_probe_tiles(c, tile, lane);
+    while (status_state(w, c.epoch) != 2u) {
+        if (scan_give_up(c, spins)) break;
+        w = scan_probe(c, tile);
     }
-    // a tile total is below 2^15 and a group accumulator below 2^21, so 32-bit sums are exact
-    uint64_t excl = wave_sum_u32((uint32_t)lane < r ? (uint32_t)pr.wt : 0u);
-    // earlier groups: back to the nearest published prefix
-    int64_t first = (int64_t)g - 1;
-    for (;;) {
-        const int64_t gi = first - lane;
-        const bool has_prefix = gi < 0 || status_state(pr.wp, c.epoch) == 2u;   // zero prefix before group 0
-        const bool complete = gi >= 0 && (uint32_t)((pr.wa >> 32) & 0xffu) == kGroupFull;
-        const uint64_t m_prefix = __ballot(has_prefix);
-        const uint64_t m_open = __ballot(!has_prefix && !complete);
-        const int stop = m_prefix ? __builtin_ctzll(m_prefix) : 64;
-        const uint64_t before = stop >= 64 ? ~0ull : ((1ull << stop) - 1ull);   // lanes that must be complete
-        if (m_open & before) {
-            if (scan_give_up(c, spins, lane)) break;
-            scan_probe_groups(c, first, lane, pr.wa, pr.wp);
-            continue;
-        }
-        excl += wave_sum_u32(lane < stop ? (uint32_t)pr.wa : 0u);
-        if (m_prefix) {
-            // the 40-bit prefix of the stopping group, read from its lane (none before group 0)
-            if (first - stop >= 0) {
-                const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)pr.wp, stop);
-                const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(pr.wp >> 32), stop);
-                excl += (((uint64_t)hi << 32) | lo) & kValueMask;
-            }
-            break;
-        }
-        first -= 64;
-        scan_probe_groups(c, first, lane, pr.wa, pr.wp);
-    }
-    if (((tile & kGroupMask) == kGroupMask || tile == c.n_tiles - 1u) && lane == 0)
-        status_store(&c.gpref[g], status_word(c.epoch, 2, excl + total));
-    return excl;
+    return w & kValueMask;
 }
 
 }  // namespace hc

@@ -12,10 +12,10 @@
 //      scan; coalesced 16-byte copy of the payload into LDS; per-lane decode
 //   3. combine: delta_out = delta_local + decoded deltas (HomComp/src/homcomp.cu:3611-3616)
 //   4a. stream output: rate selection, header bytes, tile-local scan, pack into one of two LDS
-//       buffers; the tile's offset in the stream comes from a two-level single-pass scan whose
-//       steps (publish, probe, resolve) are spread over this and the next two rounds, so the
-//       payload is copied to the stream (coalesced 16-byte stores) two rounds after it was
-//       packed and no round waits for another workgroup
+//       buffers; the tile's offset in the stream comes from the scan-server workgroup of the
+//       same launch (publish the tile total in this round, request the prefix in the next, use
+//       it in the one after), so the payload is copied to the stream (coalesced 16-byte stores)
+//       two rounds after it was packed and no data workgroup waits for another
 //   4b. float output: in-block running sum, dequantise, two float4 stores per lane
 // Small streaming kernels cover the incoming-stream offsets, the Lorenzo pre-pass and the
 // value range.
@@ -113,6 +113,68 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
 template <int OUT>
 constexpr int tile_threads() { return kWG; }
 
+// The scan server: one workgroup of the launch that turns the tile totals the data workgroups
+// publish into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  Each step covers 1024 tiles in
+// index order, 4 per lane: wait for the totals, scan, write the prefixes.  The data workgroups
+// publish a whole round (gridDim.x - 1 consecutive tiles) at about the same time, so a step
+// rarely waits long.  Also writes the stream length once the last tile is in.
+__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c)
+{
+    __shared__ uint32_t s_wave[kWG / 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    uint64_t base = 0;
+    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += kWG * 4) {
+        const uint32_t idx = t0 + (uint32_t)tid * 4u;   // n_tiles is a multiple of 8
+        const bool in = idx < c.n_tiles;
+        uint64_t w[4] = {0, 0, 0, 0};
+        if (in) {
+            uint32_t spins = 0;
+            for (;;) {
+                bool ok = true;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    w[j] = status_load(&c.totals[idx + j]);
+                    ok = ok && status_state(w[j], c.epoch) == 1u;
+                }
+                if (ok || scan_give_up(c, spins)) break;
+            }
+        }
+        uint32_t v[4], mine = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+            mine += v[j];
+        }
+        const uint32_t incl = wave_incl_scan_u32(mine, lane);
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        uint32_t before = 0, step_total = 0;
+#pragma unroll
+        for (int q = 0; q < kWG / 64; ++q) {
+            const uint32_t t = s_wave[q];
+            if (q < wave) before += t;
+            step_total += t;
+        }
+        if (in) {
+            uint64_t run = base + before + (incl - mine);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
+                run += v[j];
+            }
+        }
+        base += step_total;
+        __syncthreads();   // s_wave is reused by the next step
+    }
+    if (tid == 0) {
+        const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
+        *p.total = len;
+        if (p.user_total) *p.user_total = len;
+    }
+}
+
 template <int NIN, int LOCAL, int OUT>
 __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p)
 {
@@ -135,9 +197,16 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
     const int lane = threadIdx.x & 63;
     const int k = tid & 3;
     const int quad = tid >> 2;
-    const int64_t G = gridDim.x;
     const int64_t n_tiles = p.n_tiles;
-    const ScanCtx scan{p.tile_status, p.group_acc, p.group_prefix, p.n_tiles, p.epoch, p.spin_limit, p.error};
+    const ScanCtx scan{p.tile_totals, p.tile_prefixes, p.n_tiles, p.epoch, p.spin_limit, p.error};
+    // on the encoder the last workgroup of the grid is the scan server, the others walk the tiles
+    const int64_t G = kEnc ? (int64_t)gridDim.x - 1 : (int64_t)gridDim.x;
+    if constexpr (kEnc) {
+        if ((int64_t)blockIdx.x == G) {
+            scan_server(p, scan);
+            return;
+        }
+    }
 
     // The local operand is prefetched two rounds ahead into two register sets that the rounds
     // use alternately.  A wave's memory operations complete in issue order and s_waitcnt can only
@@ -150,9 +219,9 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
         load_local<LOCAL>(buf_b, p.local, p.n, (uint64_t)(blockIdx.x + G) * kTileElems, tid);
 
     // scan pipeline registers of wave 0: byte totals of the tiles of the previous two rounds and
-    // the probe that was issued in the previous round for the older of the two
+    // the prefix word requested in the previous round for the older of the two
     uint32_t total1 = 0, total2 = 0;
-    ScanProbe probe{0, 0, 0};
+    uint64_t probe = 0;
 
     // A round handles tile t0 (operand in `nxt`) and, on the encoder, finishes the scan and the
     // store of the tiles of the two rounds before (t1, t2).  Returns false when nothing is left.
@@ -292,7 +361,7 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
             //      operations complete in issue order, so the resolve step, which needs the probe
             //      issued a round ago, comes before this round's stores and loads of the wave.
             if (scanw && v2) {
-                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, total2, probe, lane);
+                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, probe);
                 if (lane == 0) {
                     s_base = p.hdr_bytes + excl;
                     s_total = total2;
@@ -303,9 +372,9 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
                 uint32_t total0 = 0;
                 if (v0) {
                     total0 = tile_scan(s_size, s_ofs_out, lane);
-                    scan_publish(scan, tile, total0, lane);
+                    if (lane == 0) scan_publish(scan, tile, total0);
                 }
-                if (v1) probe = scan_probe(scan, (uint32_t)t1, lane);
+                if (v1) probe = scan_probe(scan, (uint32_t)t1);
                 total2 = total1;
                 total1 = total0;
             }
@@ -315,12 +384,6 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
                 const uint64_t gofs = s_base;
                 const uint32_t tot = s_total;
                 copy_out(s_out[buf], p.out_cmp + gofs, tot, tid);
-                // true stream length = end offset of the last tile (HomComp/src/GSZ.cu:752-755)
-                if (t2 == n_tiles - 1 && tid == 0) {
-                    const uint64_t len = gofs + tot;
-                    *p.total = len;
-                    if (p.user_total) *p.user_total = len;
-                }
             }
             __syncthreads();
             // ---- the operand of the round after the next one starts to fly now
@@ -537,7 +600,11 @@ __global__ void k_fill_u64(uint64_t *p, uint64_t n)
 template <int NIN, int LOCAL, int OUT>
 static hipError_t launch_tile(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
-    const uint32_t grid = p.n_tiles < max_grid ? p.n_tiles : max_grid;
+    // encoder: data workgroups + the scan server, together no more than the device keeps resident
+    const uint32_t extra = OUT == kOutStream ? 1u : 0u;
+    uint32_t grid = p.n_tiles + extra;
+    if (grid > max_grid) grid = max_grid;
+    if (grid < 1u + extra) grid = 1u + extra;
     hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(grid), dim3(tile_threads<OUT>()), 0, s, p);
     return hipGetLastError();
 }

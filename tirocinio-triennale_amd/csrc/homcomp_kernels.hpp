@@ -14,8 +14,6 @@ enum : int { kOpCompress = 0, kOpDecompress, kOpHomSumF32, kOpHomSumI32, kOpHomA
 constexpr uint32_t kHostTileElems = 4096;
 constexpr uint32_t kHostTileBlocks = 128;
 constexpr uint32_t kHostChunkElems = 32768;
-constexpr uint32_t kHostGroupTiles = 64;
-constexpr uint32_t kHostAccStride = 16;   // 64-bit words between two group accumulators
 
 struct TileParams {
     const uint8_t *in[2];       // incoming streams (header + payload)
@@ -29,9 +27,8 @@ struct TileParams {
     uint32_t n_tiles;           // padded length / 4096
     float eb;
     float recip;                // fl(0.5f / eb), rounded on the host
-    uint64_t *tile_status;      // output-offset scan: one word per tile,
-    uint64_t *group_acc;        // one accumulator (zero at launch)
-    uint64_t *group_prefix;     // and one prefix word per group of 64 tiles
+    uint64_t *tile_totals;      // output-offset scan: per tile the byte total (data workgroups)
+    uint64_t *tile_prefixes;    // and the exclusive prefix (scan server)
     uint32_t epoch;             // tag that makes this launch's status words distinguishable
     uint32_t spin_limit;        // bound on unsuccessful scan probes before *error is raised
     uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
