@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -15,7 +16,10 @@ namespace {
 thread_local int g_last_hip_error = 0;
 
 constexpr uint32_t kMaxEpoch = (1u << 22) - 1;
-constexpr uint32_t kSpinLimit = 1u << 22;   // unsuccessful scan probes (~seconds) before giving up
+// Unsuccessful scan re-reads before a wave gives up (each costs a memory round trip, so this is
+// some tens of milliseconds): long enough for any delay of a resident workgroup, short enough
+// that a launch which could not become resident ends with an error instead of stalling for minutes.
+constexpr uint32_t kSpinLimit = 1u << 16;
 constexpr uint32_t kRangePartials = 2048;
 
 inline bool hip_ok(hipError_t e)
@@ -47,6 +51,7 @@ struct homcomp_workspace {
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
     uint32_t max_grid[hc::kOpCount];  // resident workgroups of each tile kernel on this device
+    uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
 };
 
 namespace {
@@ -82,7 +87,7 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
     p->n_tiles = (uint32_t)(padded_len(n) / hc::kHostTileElems);
     p->tile_totals = ws->d_tile_totals;
     p->tile_prefixes = ws->d_tile_prefixes;
-    p->spin_limit = kSpinLimit;
+    p->spin_limit = ws->spin_limit;
     p->error = ws->d_error;
     p->total = ws->d_total;
     return next_epoch(ws, s, &p->epoch);
@@ -183,8 +188,22 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         int per_cu = 0;
         ok = hip_ok(hc::tile_kernel_residency(op, &per_cu));
         if (ok && per_cu < 1) per_cu = 1;
-        ws->max_grid[op] = (uint32_t)per_cu * (uint32_t)prop.multiProcessorCount;
+        // one compute unit's worth of workgroups is left free: the persistent grid must be fully
+        // resident, and an estimate that is off by a single workgroup would stall the launch
+        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
+        ws->max_grid[op] = (uint32_t)per_cu * (uint32_t)cus;
+        // HOMCOMP_GRID_PERCENT (1..100) shrinks the persistent grid, for devices that are shared
+        // with other work and cannot keep a full grid of this library resident
+        if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
+            const long pct = std::strtol(e, nullptr, 10);
+            if (pct >= 1 && pct <= 100) ws->max_grid[op] = (uint32_t)((uint64_t)ws->max_grid[op] * (uint64_t)pct / 100u);
+        }
         if (ws->max_grid[op] < 2) ws->max_grid[op] = 2;   // an encoder needs a data workgroup and the scan server
+    }
+    ws->spin_limit = kSpinLimit;
+    if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {
+        const long v = std::strtol(e, nullptr, 10);
+        if (v >= 1 && v <= (1l << 30)) ws->spin_limit = (uint32_t)v;
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
         !hip_ok(hipHostMalloc((void **)&ws->h_total, 2 * sizeof(uint64_t), hipHostMallocDefault))) {
