@@ -266,3 +266,28 @@ def test_argument_errors(gpu, pkg, cuda):
     assert L.homcomp_compress_f32(None, x.data_ptr(), 64, C.c_float(1e-3), cmp.data_ptr(), None, None) == -1
     assert L.homcomp_compress_f32(h, None, 64, C.c_float(1e-3), cmp.data_ptr(), None, None) == -1
     assert pkg.status_string(-2).startswith("float")
+
+
+@pytest.mark.parametrize("grid_percent", [100, 50, 10, 1])
+def test_many_rounds_and_small_grids(pkg, cuda, orc, gen, monkeypatch, grid_percent):
+    """Inputs much larger than the persistent grid (many rounds per workgroup), for every
+    stream-producing entry point, also with the grid shrunk through HOMCOMP_GRID_PERCENT: the
+    scan server's step size has to follow the grid size or the launch stalls."""
+    monkeypatch.setenv("HOMCOMP_GRID_PERCENT", str(grid_percent))
+    n = 1 << 23 if grid_percent >= 10 else 1 << 21
+    orc.set_threads(16)
+    a, b = gen.uniform_np(n, 31), gen.smooth_np(n, 32)
+    eb = np.float32(1e-3)
+    g = Gpu(pkg, cuda, n)
+    try:
+        sa = g.compress(a, eb)
+        assert_stream_equal(sa, orc.compress(a, eb), "compress")
+        sb = g.compress(b, eb)
+        want = orc.hom_sum_f32(sa, b, eb)
+        assert_stream_equal(g.hom_sum_f32(sa, b, eb), want, "hom_sum_f32")
+        assert_stream_equal(g.hom_add(sa, sb, n), want, "hom_add")
+        assert_stream_equal(g.hom_sum_i32(sa, orc.quant_predict(b, eb)), want, "hom_sum_i32")
+        dec = g.decompress(want, n, eb)
+        assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
+    finally:
+        g.close()

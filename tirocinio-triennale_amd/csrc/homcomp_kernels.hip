@@ -114,37 +114,48 @@ template <int OUT>
 constexpr int tile_threads() { return kWG; }
 
 // The scan server: one workgroup of the launch that turns the tile totals the data workgroups
-// publish into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  Each step covers 1024 tiles in
-// index order, 4 per lane: wait for the totals, scan, write the prefixes.  The data workgroups
-// publish a whole round (gridDim.x - 1 consecutive tiles) at about the same time, so a step
+// publish into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  It sweeps the tiles in index
+// order in steps: wait for the step's totals, scan them, write the prefixes, go on.  The data
+// workgroups publish a whole round (G consecutive tiles) at about the same time, so a step
 // rarely waits long.  Also writes the stream length once the last tile is in.
-__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c)
+//
+// Step size and progress: a data workgroup uses the prefix of its round-r tile in round r+2,
+// before it publishes its round-(r+2) tile.  A step must therefore never contain both a tile and
+// the tile 2G after it (the step could not complete before the workgroup that waits for it has
+// published), i.e. a step covers at most 2G tiles: 1024 tiles (4 per lane) when G >= 512,
+// otherwise one tile per lane on min(256, 2G) lanes.
+__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
 {
     __shared__ uint32_t s_wave[kWG / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const uint32_t per = G >= 512u ? 4u : 1u;                                   // tiles per lane
+    const uint32_t lanes = G >= 512u ? (uint32_t)kWG : (2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
+    const uint32_t step = per * lanes;
     uint64_t base = 0;
-    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += kWG * 4) {
-        const uint32_t idx = t0 + (uint32_t)tid * 4u;   // n_tiles is a multiple of 8
-        const bool in = idx < c.n_tiles;
+    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += step) {
+        const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
+        const bool in = (uint32_t)tid < lanes && idx < c.n_tiles;
         uint64_t w[4] = {0, 0, 0, 0};
         if (in) {
             uint32_t spins = 0;
             for (;;) {
                 bool ok = true;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    w[j] = status_load(&c.totals[idx + j]);
-                    ok = ok && status_state(w[j], c.epoch) == 1u;
+                for (uint32_t j = 0; j < 4; ++j) {
+                    if (j < per) {
+                        w[j] = status_load(&c.totals[idx + j]);
+                        ok = ok && status_state(w[j], c.epoch) == 1u;
+                    }
                 }
                 if (ok || scan_give_up(c, spins)) break;
             }
         }
         uint32_t v[4], mine = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+        for (uint32_t j = 0; j < 4; ++j) {
+            v[j] = in && j < per ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
             mine += v[j];
         }
         const uint32_t incl = wave_incl_scan_u32(mine, lane);
@@ -160,9 +171,11 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
         if (in) {
             uint64_t run = base + before + (incl - mine);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
-                run += v[j];
+            for (uint32_t j = 0; j < 4; ++j) {
+                if (j < per) {
+                    status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
+                    run += v[j];
+                }
             }
         }
         base += step_total;
@@ -203,7 +216,7 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
     const int64_t G = kEnc ? (int64_t)gridDim.x - 1 : (int64_t)gridDim.x;
     if constexpr (kEnc) {
         if ((int64_t)blockIdx.x == G) {
-            scan_server(p, scan);
+            scan_server(p, scan, (uint32_t)G);
             return;
         }
     }
