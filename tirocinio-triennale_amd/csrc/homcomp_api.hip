@@ -44,7 +44,8 @@ struct homcomp_workspace {
     uint64_t *d_tile_totals;   // [max_tiles]  output-offset scan: tile totals
     uint64_t *d_tile_prefixes; // [max_tiles]  output-offset scan: tile prefixes (adjacent to the totals)
     uint64_t *d_in_ofs[2];    // [max_tiles+1] tile payload offsets of the incoming streams
-    uint32_t *d_in_totals;    // [max_tiles]   scratch of the offsets pre-pass
+    uint32_t *d_in_totals;    // [max_tiles]   scratch of the offsets pre-pass: tile totals
+    uint32_t *d_in_blocks;    // [max_tiles/256 + 1]  and sums over blocks of 256 tiles
     uint64_t *d_total;        // stream length of the last stream-producing call
     uint32_t *d_error;        // sticky error flags, next to d_total
     float *d_partial;         // min/max partials
@@ -97,7 +98,8 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
 int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::TileParams *p, hipStream_t s)
 {
     p->in_ofs[c] = ws->d_in_ofs[c];
-    return hip_ok(hc::launch_in_offsets(d_cmp, p->n_tiles, p->hdr_bytes, ws->d_in_totals, ws->d_in_ofs[c], s))
+    return hip_ok(hc::launch_in_offsets(d_cmp, p->n_tiles, p->hdr_bytes, ws->d_in_totals, ws->d_in_blocks,
+                                        ws->d_in_ofs[c], s))
                ? HOMCOMP_OK
                : HOMCOMP_ERR_HIP;
 }
@@ -179,6 +181,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     const size_t o_in0 = take((t + 1) * sizeof(uint64_t));
     const size_t o_in1 = take((t + 1) * sizeof(uint64_t));
     const size_t o_tot = take(t * sizeof(uint32_t));
+    const size_t o_blk = take((t / 256 + 1) * sizeof(uint32_t));
     const size_t o_total = take(64);
     const size_t o_partial = take(kRangePartials * 2 * sizeof(float));
     const size_t bytes = off;
@@ -199,6 +202,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
             if (pct >= 1 && pct <= 100) ws->max_grid[op] = (uint32_t)((uint64_t)ws->max_grid[op] * (uint64_t)pct / 100u);
         }
         if (ws->max_grid[op] < 2) ws->max_grid[op] = 2;   // an encoder needs a data workgroup and the scan server
+        // decompression has no dependence between tiles: one workgroup per tile, scheduled by the hardware
+        if (op == hc::kOpDecompress) ws->max_grid[op] = 0x7fffffffu;
     }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {
@@ -217,6 +222,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     ws->d_in_ofs[0] = (uint64_t *)(base + o_in0);
     ws->d_in_ofs[1] = (uint64_t *)(base + o_in1);
     ws->d_in_totals = (uint32_t *)(base + o_tot);
+    ws->d_in_blocks = (uint32_t *)(base + o_blk);
     ws->d_total = (uint64_t *)(base + o_total);
     ws->d_error = (uint32_t *)(base + o_total + 8);
     ws->d_partial = (float *)(base + o_partial);

@@ -423,80 +423,99 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
 // ---------------------------------------------------------------- incoming-stream offsets
 //
 // The payload offset of a tile of an incoming stream depends on the header bytes only
-// (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel: k_in_totals sums
-// the block sizes of every tile (8 lanes per tile, 16 header bytes per lane), k_in_scan turns
-// the totals into exclusive offsets (one workgroup; `base` = header length is added).
+// (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel in two fully parallel
+// steps over blocks of 256 tiles: k_in_totals sums the block sizes of every tile (8 lanes per
+// tile, 16 header bytes per lane) and leaves one sum per block; k_in_offsets adds up the sums of
+// the earlier blocks, scans the block's 256 totals and writes the tiles' absolute offsets
+// (`base` = header length).
 
-__global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ hdr, uint32_t n_tiles,
-                                                   uint32_t *__restrict__ totals)
+constexpr uint32_t kOfsBlockTiles = 256;
+
+__device__ __forceinline__ uint32_t wg_reduce_u32(uint32_t v, uint32_t *s_tmp)
 {
-    const uint32_t t = blockIdx.x * 256u + threadIdx.x;   // 16-byte piece index
-    const uint32_t tile = t >> 3;
-    uint32_t sum = 0;
-    if (tile < n_tiles) {
-        const uint8_t *src = hdr + (uint64_t)t * 16u;
-        uint32_t w[4];
-        if (((uintptr_t)src & 15u) == 0) {
-            const uint4 q = *reinterpret_cast<const uint4 *>(src);
-            w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                w[i] = (uint32_t)src[4 * i] | ((uint32_t)src[4 * i + 1] << 8) |
-                       ((uint32_t)src[4 * i + 2] << 16) | ((uint32_t)src[4 * i + 3] << 24);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int b = 0; b < 4; ++b) sum += size_from_header((w[i] >> (8 * b)) & 0xffu);
-    }
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    sum += __shfl_xor(sum, 4, 64);
-    if (tile < n_tiles && (threadIdx.x & 7) == 0) totals[tile] = sum;
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = v;
+    __syncthreads();
+    uint32_t t = 0;
+    for (uint32_t w = 0; w < blockDim.x / 64; ++w) t += s_tmp[w];
+    __syncthreads();
+    return t;
 }
 
-__global__ __launch_bounds__(1024) void k_in_scan(const uint32_t *__restrict__ totals, uint32_t n_tiles,
-                                                  uint64_t base, uint64_t *__restrict__ ofs)
+__global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ hdr, uint32_t n_tiles,
+                                                   uint32_t *__restrict__ totals,
+                                                   uint32_t *__restrict__ block_sums)
 {
-    // Each thread owns a contiguous run of `per` tiles (a multiple of 4, read as 16-byte
-    // vectors with all loads of a pass in flight together); n_tiles is a multiple of 8.
-    __shared__ uint64_t s_part[1024];
-    constexpr uint32_t kVec = 4, kUnroll = 4;
-    const uint32_t per = (((n_tiles + 1023u) / 1024u) + kVec - 1u) / kVec * kVec;
-    const uint32_t lo = threadIdx.x * per;
-    const uint32_t hi = lo + per < n_tiles ? lo + per : n_tiles;   // lo, hi multiples of 4 (or lo >= hi)
-    uint64_t sum = 0;
-    for (uint32_t i = lo; i < hi; i += kVec * kUnroll) {
-        u32x4 q[kUnroll];
+    __shared__ uint32_t s_tmp[4];
+    uint32_t acc = 0;
+    for (uint32_t it = 0; it < kOfsBlockTiles / 32; ++it) {
+        // 16-byte piece index: 8 pieces per tile, 32 tiles per pass of the workgroup
+        const uint32_t t = (blockIdx.x * (kOfsBlockTiles / 32) + it) * 256u + threadIdx.x;
+        const uint32_t tile = t >> 3;
+        uint32_t sum = 0;
+        if (tile < n_tiles) {
+            const uint8_t *src = hdr + (uint64_t)t * 16u;
+            uint32_t w[4];
+            if (((uintptr_t)src & 15u) == 0) {
+                const u32x4 q = *reinterpret_cast<const u32x4 *>(src);
+                w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+            } else {
 #pragma unroll
-        for (uint32_t u = 0; u < kUnroll; ++u)
-            q[u] = i + u * kVec < hi ? *reinterpret_cast<const u32x4 *>(totals + i + u * kVec) : u32x4{0, 0, 0, 0};
+                for (int i = 0; i < 4; ++i)
+                    w[i] = (uint32_t)src[4 * i] | ((uint32_t)src[4 * i + 1] << 8) |
+                           ((uint32_t)src[4 * i + 2] << 16) | ((uint32_t)src[4 * i + 3] << 24);
+            }
 #pragma unroll
-        for (uint32_t u = 0; u < kUnroll; ++u) sum += (uint64_t)q[u].x + q[u].y + q[u].z + q[u].w;
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) sum += size_from_header((w[i] >> (8 * b)) & 0xffu);
+        }
+        acc += sum;
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        if (tile < n_tiles && (threadIdx.x & 7) == 0) totals[tile] = sum;
     }
-    s_part[threadIdx.x] = sum;
+    const uint32_t block_total = wg_reduce_u32(acc, s_tmp);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total;
+}
+
+__global__ __launch_bounds__(256) void k_in_offsets(const uint32_t *__restrict__ totals,
+                                                    const uint32_t *__restrict__ block_sums,
+                                                    uint32_t n_tiles, uint64_t base,
+                                                    uint64_t *__restrict__ ofs)
+{
+    __shared__ uint32_t s_tmp[4];
+    __shared__ uint32_t s_wave[4];
+    // bytes of all earlier blocks (a block is at most 256 * 132 * 128 bytes, so 64-bit sums)
+    uint64_t before = 0;
+    for (uint32_t q0 = 0; q0 < blockIdx.x; q0 += 256) {
+        const uint32_t q = q0 + threadIdx.x;
+        const uint32_t v = q < blockIdx.x ? block_sums[q] : 0u;
+        // split so that the 32-bit reduction cannot overflow (256 values below 2^23 each)
+        before += (uint64_t)wg_reduce_u32(v & 0xffffu, s_tmp) + ((uint64_t)wg_reduce_u32(v >> 16, s_tmp) << 16);
+    }
+    const uint32_t tile = blockIdx.x * kOfsBlockTiles + threadIdx.x;
+    const uint32_t mine = tile < n_tiles ? totals[tile] : 0u;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t incl = wave_incl_scan_u32(mine, lane);
+    if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
-    // Hillis-Steele inclusive scan of the 1024 partial sums
-    for (uint32_t d = 1; d < 1024; d <<= 1) {
-        const uint64_t add = threadIdx.x >= d ? s_part[threadIdx.x - d] : 0;
-        __syncthreads();
-        s_part[threadIdx.x] += add;
-        __syncthreads();
-    }
-    uint64_t run = base + s_part[threadIdx.x] - sum;
-    for (uint32_t i = lo; i < hi; i += kVec) {
-        const u32x4 q = *reinterpret_cast<const u32x4 *>(totals + i);
-        uint64_t o[4];
-        o[0] = run;
-        o[1] = o[0] + q.x;
-        o[2] = o[1] + q.y;
-        o[3] = o[2] + q.z;
-        run = o[3] + q.w;
+    uint32_t earlier = 0, block_total = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) ofs[i + j] = o[j];
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t t = s_wave[q];
+        if (q < wave) earlier += t;
+        block_total += t;
     }
-    if (threadIdx.x == 1023) ofs[n_tiles] = base + s_part[1023];
+    if (tile < n_tiles) ofs[tile] = base + before + earlier + (incl - mine);
+    // the entry after the last tile is the end of the payload
+    if (threadIdx.x == 0 && (blockIdx.x + 1) * kOfsBlockTiles >= n_tiles) ofs[n_tiles] = base + before + block_total;
 }
 
 // HomComp/src/homcomp.cu:1553-1602: Lorenzo deltas of the quantised values as int32.
@@ -654,11 +673,11 @@ hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStr
 }
 
 hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
-                             uint64_t *ofs, hipStream_t s)
+                             uint32_t *block_sums, uint64_t *ofs, hipStream_t s)
 {
-    const uint32_t pieces = n_tiles * 8u;
-    hipLaunchKernelGGL(k_in_totals, dim3((pieces + 255u) / 256u), dim3(256), 0, s, hdr, n_tiles, totals);
-    hipLaunchKernelGGL(k_in_scan, dim3(1), dim3(1024), 0, s, totals, n_tiles, base, ofs);
+    const uint32_t blocks = (n_tiles + kOfsBlockTiles - 1) / kOfsBlockTiles;
+    hipLaunchKernelGGL(k_in_totals, dim3(blocks), dim3(256), 0, s, hdr, n_tiles, totals, block_sums);
+    hipLaunchKernelGGL(k_in_offsets, dim3(blocks), dim3(256), 0, s, totals, block_sums, n_tiles, base, ofs);
     return hipGetLastError();
 }
 

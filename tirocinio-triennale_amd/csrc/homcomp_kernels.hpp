@@ -41,7 +41,7 @@ hipError_t tile_kernel_residency(int op, int *blocks_per_cu);
 hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
 // Tile payload offsets of an incoming stream from its header bytes.
 hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
-                             uint64_t *ofs, hipStream_t s);
+                             uint32_t *block_sums, uint64_t *ofs, hipStream_t s);
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s);
 hipError_t launch_range(const float *x, uint64_t n, float *partial, uint32_t max_partials,
                         float *out, hipStream_t s);
