@@ -24,6 +24,11 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X published peak
 
+# HBM bytes per launch of the dominant kernel (hom_sum_f32) measured with rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE and scaled as described in profiles/pmc_hbm_traffic_smooth_1GiB_rel1e-4.txt;
+# keyed by (kind, log2n, rel).  Other workloads report null.
+MEASURED_TRAFFIC = {("smooth", 28, 1e-4): 1.3647e9}
+
 
 def time_op(torch, fn, iters: int) -> float:
     """Average kernel-side milliseconds per call, HIP events on the launch stream."""
@@ -158,7 +163,7 @@ def main() -> int:
     dom = "hom_sum_f32"
     roofline = {"bound": "hbm", "kernel": dom, "achieved": ops[dom]["achieved_GBps"],
                 "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ops[dom]["frac_hbm"],
-                "traffic": None}
+                "traffic": MEASURED_TRAFFIC.get((args.kind, args.log2n, args.rel)) if args.abs is None else None}
 
     out = {
         "metric": "compress + hom-add throughput (GB/s of uncompressed input)",
