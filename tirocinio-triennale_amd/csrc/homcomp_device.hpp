@@ -11,12 +11,14 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "homcomp_kernels.hpp"
+
 namespace hc {
 
 constexpr int kWG = 256;                              // threads per workgroup (4 waves)
 constexpr int kEPL = 8;                               // elements per lane per iteration
 constexpr int kQuad = 4;                              // lanes per 32-element block
-constexpr int kIter = 2;                              // iterations per tile
+constexpr int kIter = HC_ITER;                        // iterations per tile
 constexpr int kBlocksPerIter = kWG / kQuad;           // 64
 constexpr int kTileBlocks = kBlocksPerIter * kIter;   // 128
 constexpr int kTileElems = kTileBlocks * 32;          // 4096

@@ -24,16 +24,25 @@
 
 namespace hc {
 
-// Tile-local exclusive scan of the 128 block sizes, run by wave 0; returns the tile total in
-// every lane.
+// Tile-local exclusive scan of the block sizes of a tile, run by one wave; returns the tile
+// total in every lane.
 __device__ __forceinline__ uint32_t tile_scan(const uint32_t *s_size, uint32_t *s_ofs, int lane)
 {
-    const uint32_t s0 = s_size[2 * lane], s1 = s_size[2 * lane + 1];
-    const uint32_t incl = wave_incl_scan_u32(s0 + s1, lane);
-    const uint32_t excl = incl - (s0 + s1);
-    s_ofs[2 * lane] = excl;
-    s_ofs[2 * lane + 1] = excl + s0;
-    return __shfl(incl, 63, 64);
+    constexpr int kPer = kTileBlocks / 64;   // blocks per lane
+    uint32_t sz[kPer], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        sz[j] = s_size[kPer * lane + j];
+        sum += sz[j];
+    }
+    const uint32_t incl = wave_incl_scan_u32(sum, lane);
+    uint32_t run = incl - sum;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        s_ofs[kPer * lane + j] = run;
+        run += sz[j];
+    }
+    return (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
 }
 
 // Registers holding one tile's share of the local operand.
@@ -134,22 +143,30 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
     const uint32_t lanes = G >= 512u ? (uint32_t)kWG : (2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
     const uint32_t step = per * lanes;
     uint64_t base = 0;
-    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += step) {
+    // The totals of a step are requested two steps ahead, into two register sets used
+    // alternately: in the steady state they were published a round ago, so the server runs at the
+    // pace of its arithmetic instead of one memory round trip per step.  Lanes beyond the end
+    // request the last tiles again (no branch around the loads) and ignore what they get.
+    const uint32_t last = c.n_tiles - per;
+    auto request = [&](uint32_t t0, uint64_t (&dst)[4]) __attribute__((always_inline)) {
+        uint32_t idx = t0 + (uint32_t)tid * per;
+        if (idx > last) idx = last;
+        for (uint32_t j = 0; j < per; ++j) dst[j] = status_load(&c.totals[idx + j]);
+    };
+    auto process = [&](uint32_t t0, uint64_t (&w)[4]) __attribute__((always_inline)) {
         const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
         const bool in = (uint32_t)tid < lanes && idx < c.n_tiles;
-        uint64_t w[4] = {0, 0, 0, 0};
         if (in) {
             uint32_t spins = 0;
             for (;;) {
                 bool ok = true;
 #pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) {
-                    if (j < per) {
-                        w[j] = status_load(&c.totals[idx + j]);
-                        ok = ok && status_state(w[j], c.epoch) == 1u;
-                    }
-                }
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (j < per) ok = ok && status_state(w[j], c.epoch) == 1u;
                 if (ok || scan_give_up(c, spins)) break;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (j < per) w[j] = status_load(&c.totals[idx + j]);
             }
         }
         uint32_t v[4], mine = 0;
@@ -180,6 +197,16 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
         }
         base += step_total;
         __syncthreads();   // s_wave is reused by the next step
+    };
+    uint64_t wa[4] = {0, 0, 0, 0}, wb[4] = {0, 0, 0, 0};
+    request(0, wa);
+    request(step, wb);
+    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += 2 * step) {
+        process(t0, wa);
+        request(t0 + 2 * step, wa);
+        if (t0 + step >= c.n_tiles) break;
+        process(t0 + step, wb);
+        request(t0 + 3 * step, wb);
     }
     if (tid == 0) {
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
@@ -424,8 +451,8 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
 //
 // The payload offset of a tile of an incoming stream depends on the header bytes only
 // (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel in two fully parallel
-// steps over blocks of 256 tiles: k_in_totals sums the block sizes of every tile (8 lanes per
-// tile, 16 header bytes per lane) and leaves one sum per block; k_in_offsets adds up the sums of
+// steps over blocks of 256 tiles: k_in_totals sums the block sizes of every tile (16 header
+// bytes per lane) and leaves one sum per block; k_in_offsets adds up the sums of
 // the earlier blocks, scans the block's 256 totals and writes the tiles' absolute offsets
 // (`base` = header length).
 
@@ -453,10 +480,11 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
 {
     __shared__ uint32_t s_tmp[4];
     uint32_t acc = 0;
-    for (uint32_t it = 0; it < kOfsBlockTiles / 32; ++it) {
-        // 16-byte piece index: 8 pieces per tile, 32 tiles per pass of the workgroup
-        const uint32_t t = (blockIdx.x * (kOfsBlockTiles / 32) + it) * 256u + threadIdx.x;
-        const uint32_t tile = t >> 3;
+    constexpr uint32_t kPieces = kTileBlocks / 16;            // 16-byte header pieces (lanes) per tile
+    constexpr uint32_t kPasses = kOfsBlockTiles * kPieces / 256;
+    for (uint32_t it = 0; it < kPasses; ++it) {
+        const uint32_t t = (blockIdx.x * kPasses + it) * 256u + threadIdx.x;   // piece index
+        const uint32_t tile = t / kPieces;
         uint32_t sum = 0;
         if (tile < n_tiles) {
             const uint8_t *src = hdr + (uint64_t)t * 16u;
@@ -476,10 +504,9 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
                 for (int b = 0; b < 4; ++b) sum += size_from_header((w[i] >> (8 * b)) & 0xffu);
         }
         acc += sum;
-        sum += __shfl_xor(sum, 1, 64);
-        sum += __shfl_xor(sum, 2, 64);
-        sum += __shfl_xor(sum, 4, 64);
-        if (tile < n_tiles && (threadIdx.x & 7) == 0) totals[tile] = sum;
+#pragma unroll
+        for (uint32_t d = 1; d < kPieces; d <<= 1) sum += __shfl_xor(sum, d, 64);
+        if (tile < n_tiles && (threadIdx.x & (kPieces - 1)) == 0) totals[tile] = sum;
     }
     const uint32_t block_total = wg_reduce_u32(acc, s_tmp);
     if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total;

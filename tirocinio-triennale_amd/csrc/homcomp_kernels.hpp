@@ -10,9 +10,13 @@ enum : int { kLocalNone = 0, kLocalF32 = 1, kLocalI32 = 2 };   // local operand 
 enum : int { kOutStream = 0, kOutF32 = 1 };                    // what a tile produces
 enum : int { kOpCompress = 0, kOpDecompress, kOpHomSumF32, kOpHomSumI32, kOpHomAdd, kOpCount };
 
-// Geometry shared with the host (must match homcomp_device.hpp).
-constexpr uint32_t kHostTileElems = 4096;
-constexpr uint32_t kHostTileBlocks = 128;
+// Tile geometry, shared by host and device: a workgroup of 256 lanes handles 8 elements per lane
+// per iteration.
+#ifndef HC_ITER
+#define HC_ITER 2
+#endif
+constexpr uint32_t kHostTileElems = 256u * 8u * HC_ITER;
+constexpr uint32_t kHostTileBlocks = kHostTileElems / 32u;
 constexpr uint32_t kHostChunkElems = 32768;
 
 struct TileParams {
