@@ -151,7 +151,12 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
     auto request = [&](uint32_t t0, uint64_t (&dst)[4]) __attribute__((always_inline)) {
         uint32_t idx = t0 + (uint32_t)tid * per;
         if (idx > last) idx = last;
-        for (uint32_t j = 0; j < per; ++j) dst[j] = status_load(&c.totals[idx + j]);
+        dst[0] = status_load(&c.totals[idx]);
+        if (per == 4u) {
+            dst[1] = status_load(&c.totals[idx + 1]);
+            dst[2] = status_load(&c.totals[idx + 2]);
+            dst[3] = status_load(&c.totals[idx + 3]);
+        }
     };
     auto process = [&](uint32_t t0, uint64_t (&w)[4]) __attribute__((always_inline)) {
         const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
@@ -159,14 +164,12 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
         if (in) {
             uint32_t spins = 0;
             for (;;) {
-                bool ok = true;
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j)
-                    if (j < per) ok = ok && status_state(w[j], c.epoch) == 1u;
+                bool ok = status_state(w[0], c.epoch) == 1u;
+                if (per == 4u)
+                    ok = ok && status_state(w[1], c.epoch) == 1u && status_state(w[2], c.epoch) == 1u &&
+                         status_state(w[3], c.epoch) == 1u;
                 if (ok || scan_give_up(c, spins)) break;
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j)
-                    if (j < per) w[j] = status_load(&c.totals[idx + j]);
+                request(t0, w);
             }
         }
         uint32_t v[4], mine = 0;
