@@ -53,6 +53,8 @@ struct homcomp_workspace {
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
     uint32_t max_grid[hc::kOpCount];  // resident workgroups of each tile kernel on this device
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
+    uint32_t wave_grid[hc::kOpCount]; // resident workgroups of each wave kernel (0: none)
+    uint8_t *d_spill;         // spill slots of the wave kernels
 };
 
 namespace {
@@ -104,8 +106,12 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
                : HOMCOMP_ERR_HIP;
 }
 
-int run_tile_op(homcomp_workspace *ws, int op, const hc::TileParams &p, hipStream_t s)
+int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, hipStream_t s)
 {
+    if (ws->wave_grid[op]) {
+        p.spill = ws->d_spill;
+        return hip_ok(hc::launch_wave_op(op, p, ws->wave_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    }
     return hip_ok(hc::launch_tile_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -205,6 +211,30 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         // decompression has no dependence between tiles: one workgroup per tile, scheduled by the hardware
         if (op == hc::kOpDecompress) ws->max_grid[op] = 0x7fffffffu;
     }
+    uint32_t max_wave_grid = 0;
+    // Kernel family: the wave-autonomous kernels; HOMCOMP_KERNELS=tile selects the
+    // workgroup-tiled kernels instead (kept for comparisons).
+    const char *family = std::getenv("HOMCOMP_KERNELS");
+    const bool use_wave = !(family && std::strcmp(family, "tile") == 0);
+    for (int op = 0; ok && use_wave && op < hc::kOpCount; ++op) {
+        int per_cu = 0;
+        ok = hip_ok(hc::wave_kernel_residency(op, &per_cu));
+        if (!ok || per_cu < 1) continue;
+        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
+        ws->wave_grid[op] = (uint32_t)per_cu * (uint32_t)cus;
+        if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
+            const long pct = std::strtol(e, nullptr, 10);
+            if (pct >= 1 && pct <= 100) ws->wave_grid[op] = (uint32_t)((uint64_t)ws->wave_grid[op] * (uint64_t)pct / 100u);
+        }
+        if (ws->wave_grid[op] < 2) ws->wave_grid[op] = 2;
+        if (ws->wave_grid[op] > max_wave_grid) max_wave_grid = ws->wave_grid[op];
+    }
+    if (ok && max_wave_grid) {
+        // two slots per data wave, no more waves than tiles
+        size_t waves = (size_t)(max_wave_grid - 1) * 4;
+        if (waves > ws->max_tiles) waves = ws->max_tiles;
+        ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 2 * hc::kSpillSlotBytes));
+    }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {
         const long v = std::strtol(e, nullptr, 10);
@@ -213,6 +243,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
         !hip_ok(hipHostMalloc((void **)&ws->h_total, 2 * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
+        if (ws->d_spill) (void)hipFree(ws->d_spill);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
@@ -236,6 +267,7 @@ int homcomp_workspace_destroy(homcomp_workspace *ws)
     int rc = HOMCOMP_OK;
     if (!hip_ok(hipDeviceSynchronize())) rc = HOMCOMP_ERR_HIP;
     if (!hip_ok(hipFree(ws->d_block))) rc = HOMCOMP_ERR_HIP;
+    if (ws->d_spill && !hip_ok(hipFree(ws->d_spill))) rc = HOMCOMP_ERR_HIP;
     if (!hip_ok(hipHostFree(ws->h_total))) rc = HOMCOMP_ERR_HIP;
     delete ws;
     return rc;

@@ -40,6 +40,14 @@ __device__ __forceinline__ V stream_load(const void *p)
 {
     return __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
 }
+// Same from a device address computed as an integer: the global address space is stated, so
+// the access is a global load, not a flat one (flat accesses count against both memory counters
+// and keep the compiler from waiting for individual loads).
+template <typename V>
+__device__ __forceinline__ V stream_load_global(uintptr_t addr)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) V *>(addr));
+}
 template <typename V>
 __device__ __forceinline__ void stream_store(void *p, V v)
 {
@@ -177,7 +185,13 @@ __device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8
 // Encoder back end for one lane (HomComp/src/GSZ.cu:245-751): writes this lane's share of the
 // block payload into the LDS stage at `pos0` (the block's tile-relative offset).  Lane k
 // contributes byte k of the sign word and of every plane; lane 0 also writes the outlier bytes.
-__device__ __forceinline__ void pack8(uint8_t *stage, uint32_t pos0, uint32_t hdr, int k,
+// `stage` may carry an explicit address space (lds_bytes / global_bytes below) so that two calls
+// with different destinations cannot be merged into one sequence of flat stores.
+typedef __attribute__((address_space(3))) uint8_t *lds_bytes;
+typedef __attribute__((address_space(1))) uint8_t *global_bytes;
+
+template <typename Bytes>
+__device__ __forceinline__ void pack8(Bytes stage, uint32_t pos0, uint32_t hdr, int k,
                                       uint32_t a[8], uint32_t sb)
 {
     const uint32_t sel = hdr >> 7;

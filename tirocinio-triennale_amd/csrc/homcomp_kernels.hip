@@ -95,6 +95,7 @@ __device__ __forceinline__ void load_local(LocalRegs<LOCAL> &r, const void *loca
 // Coalesced copy of a packed tile payload from LDS to its (arbitrarily aligned) place in the
 // stream: bytes up to the first 16-byte boundary, aligned 16-byte stores assembled from
 // unaligned LDS words with v_alignbyte, then the remaining bytes.
+template <int LANES = kWG>
 __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint32_t tot, int tid)
 {
     const uint32_t mis = (uint32_t)((uintptr_t)g & 15u);
@@ -105,7 +106,7 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
     const uint32_t tail = body & 15u;
     if ((uint32_t)tid < head) g[tid] = stage[tid];
     const uint32_t *sw = reinterpret_cast<const uint32_t *>(stage);
-    for (uint32_t c = tid; c < nch; c += kWG) {
+    for (uint32_t c = tid; c < nch; c += LANES) {
         const uint32_t s = head + 16u * c;
         const uint32_t w0 = s >> 2, sh = s & 3u;
         const uint32_t x0 = sw[w0], x1 = sw[w0 + 1], x2 = sw[w0 + 2], x3 = sw[w0 + 3], x4 = sw[w0 + 4];
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
                 for (uint32_t i = (uint32_t)tid; i < nchunks; i += kWG) {
                     if (16u * (i + 1u) <= nbytes) {
                         *reinterpret_cast<u32x4 *>(&s_in[c][16u * i]) =
-                            stream_load<u32x4>(reinterpret_cast<const void *>(ga + 16u * (uintptr_t)i));
+                            stream_load_global<u32x4>(ga + 16u * (uintptr_t)i);
                     } else {
                         for (uint32_t j = 16u * i; j < nbytes; ++j)
                             s_in[c][j] = *reinterpret_cast<const uint8_t *>(ga + j);
@@ -447,6 +448,408 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
     for (int64_t t0 = blockIdx.x;; t0 += 2 * G) {
         if (!round(t0, buf_a)) break;
         if (!round(t0 + G, buf_b)) break;
+    }
+}
+
+
+// ---------------------------------------------------------------- wave-autonomous kernels
+//
+// k_wave<NIN, LOCAL, OUT>: all five operations with one tile per WAVE and no workgroup barrier
+// anywhere.  A workgroup is four independent waves that share nothing but the launch; each wave
+// walks its tiles (tile = wave index, += number of data waves) and handles a tile as kSub
+// sub-steps of 16 blocks (512 elements, 8 per lane, 4 lanes per block).  Everything a sub-step
+// consumes from memory was requested two sub-steps earlier into registers (two register sets
+// used alternately), across tile boundaries as well:
+//   local operand      2 x 16 bytes per lane
+//   incoming payload   the 16 blocks of a sub-step are one contiguous byte range of the stream;
+//                      lane l holds its l-th aligned 16-byte chunk (ranges beyond 1 KiB fetch the
+//                      rest on the spot), which goes through a small LDS stage to the byte-wise
+//                      decoder
+//   incoming headers   the 128 header bytes of the next tile are fetched a tile ahead; before the
+//                      first payload request of that tile they are turned into block offsets
+//                      (in-wave scan) and kept in LDS, double-buffered by tile parity
+// Stream output: rate selection, an in-wave DPP scan of the 16 block sizes, pack at the running
+// offset into the wave's LDS stage.  The tile's place in the stream comes from the scan server
+// (HomComp/src/GSZ.cu:170-239): total published when the tile is packed, prefix requested a
+// round later, payload copied out two rounds later.  The LDS stage of a deferred tile holds
+// wave_cap() bytes (the budget that lets 12-16 waves share a compute unit); a tile that outgrows
+// it continues in the wave's slot of a global spill area and is copied out from there.
+constexpr int kSub = kTileBlocks / 16;
+constexpr int kInStage = 16 * kMaxBlockBytes + 48;   // one sub-step's payload range plus alignment slack
+
+template <int NIN>
+constexpr int wave_cap() { return NIN == 0 ? 4096 : (NIN == 1 ? 3072 : 2048); }
+
+template <int LOCAL>
+struct SubRegs {
+    f32x4 f[2];
+    i32x4 i[2];
+};
+
+// Buffer addressing: the descriptor (base, byte count) lives in scalar registers, a lane adds a
+// constant offset, and the hardware checks every dword against the byte count: loads beyond it
+// return 0 and stores beyond it are dropped.  So the ends of the buffers need no branches, a
+// request is a fixed number of memory operations (which lets the compiler wait for exactly the
+// request it needs), and no per-lane address arithmetic is left.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, uint64_t bytes)
+{
+    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+constexpr int kBufNt = 2;   // cache policy bits of the buffer builtins: non-temporal
+
+// Operand of one sub-step of the tile whose elements start at `tile_elem0` (beyond n: zeros).
+template <int LOCAL>
+__device__ __forceinline__ void load_sub(SubRegs<LOCAL> &r, const void *local, uint64_t n, uint64_t tile_elem0,
+                                         bool valid, int s, int lane)
+{
+    if constexpr (LOCAL == kLocalNone) return;
+    const uint64_t left = valid && tile_elem0 < n ? (n - tile_elem0) * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t rs = buffer_of((const uint8_t *)local + (valid ? tile_elem0 * 4u : 0u), left);
+    const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32, s * 2048, kBufNt);
+    const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32 + 16, s * 2048, kBufNt);
+    if constexpr (LOCAL == kLocalF32) {
+        r.f[0] = __builtin_bit_cast(f32x4, a);
+        r.f[1] = __builtin_bit_cast(f32x4, b);
+    } else {
+        r.i[0] = __builtin_bit_cast(i32x4, a);
+        r.i[1] = __builtin_bit_cast(i32x4, b);
+    }
+}
+
+// Orders the LDS traffic of the lanes of one wave: LDS operations of a wave execute in program
+// order, so no instruction is needed, only a point the compiler does not move them across.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Copy of a spilled tile from the wave's slot of the spill area to its place in the stream.  The
+// slot is read with device-scope loads (it was written by this wave, but an older copy of the
+// line may sit in the vector cache from the slot's previous use).
+__device__ __forceinline__ void copy_out_spill(const uint8_t *slot, uint8_t *g, uint32_t tot, int lane)
+{
+    const uint32_t mis = (uint32_t)((uintptr_t)g & 3u);
+    uint32_t head = (4u - mis) & 3u;
+    if (head > tot) head = tot;
+    const uint32_t *sw = reinterpret_cast<const uint32_t *>(slot);
+    auto word = [&](uint32_t w) { return __hip_atomic_load(sw + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    if ((uint32_t)lane < head) g[lane] = (uint8_t)(word(0) >> (8 * lane));
+    const uint32_t nw = (tot - head) >> 2;
+    const uint32_t tail = (tot - head) & 3u;
+    const uint32_t sh = head & 3u;
+    for (uint32_t c = lane; c < nw; c += 64) {
+        const uint32_t s = head + 4u * c;
+        const uint32_t w0 = s >> 2;
+        const uint32_t x0 = word(w0), x1 = word(w0 + 1);
+        *reinterpret_cast<uint32_t *>(g + s) = __builtin_amdgcn_alignbyte(x1, x0, sh);
+    }
+    if ((uint32_t)lane < tail) {
+        const uint32_t s = head + 4u * nw + lane;
+        g[s] = (uint8_t)(word(s >> 2) >> (8 * (s & 3u)));
+    }
+}
+
+// Registers of one incoming stream that travel ahead of the computation.
+struct InRegs {
+    u32x4 chunk;   // the lane's 16-byte chunk of a sub-step's payload range
+};
+
+template <int NIN, int LOCAL, int OUT>
+__global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
+{
+    constexpr bool kEnc = OUT == kOutStream;
+    constexpr int kW = kWG / 64;
+    constexpr int kIn = NIN > 0 ? NIN : 1;
+    constexpr int kCap = wave_cap<NIN>();
+    // Sub-steps between a request and its use.  A wave's memory operations complete in order, so
+    // waiting for a load also waits for every store issued before it: the decoder, which stores
+    // 2 KiB per sub-step, looks further ahead to keep more of its stores in flight.
+    constexpr int kDepth = kEnc ? 2 : 4;
+    static_assert(kSub % kDepth == 0, "the register sets rotate with the sub-steps of a tile");
+    __shared__ __align__(16) uint8_t s_out[kW][2][kEnc ? kCap + 64 : 16];
+    __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
+    __shared__ __align__(16) uint8_t s_in[kW][kIn][NIN > 0 ? kInStage : 16];
+    __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
+    __shared__ __align__(4) uint8_t s_hdr_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 4];
+    __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512];     // decoder: exchange of the lanes' output pieces
+    __shared__ uint32_t s_rel[kW][kIn][2][NIN > 0 ? kSub + 1 : 1];   // tile-relative start of every sub-step's range
+
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave-uniform, kept in a scalar register
+    const int lane = threadIdx.x & 63;
+    const int k = lane & 3;
+    const int quad = lane >> 2;
+    const int64_t n_tiles = p.n_tiles;
+    const ScanCtx scan{p.tile_totals, p.tile_prefixes, p.n_tiles, p.epoch, p.spin_limit, p.error};
+    // on the encoder the last workgroup of the grid is the scan server
+    const int64_t G = kEnc ? (int64_t)gridDim.x - 1 : (int64_t)gridDim.x;
+    const int64_t GW = G * kW;   // data waves
+    if constexpr (kEnc) {
+        if ((int64_t)blockIdx.x == G) {
+            scan_server(p, scan, (uint32_t)(GW < 0x7fffffff ? GW : 0x7fffffff));
+            return;
+        }
+    }
+    const int64_t wid = (int64_t)blockIdx.x * kW + wave;
+    if (wid >= n_tiles) return;   // no barrier in this kernel: a wave without work just leaves
+
+    auto tile_of = [&](int64_t r) { return wid + r * GW; };
+
+    // ---- incoming streams: per-tile context
+    uint32_t hdr_next[kIn];     // header bytes of blocks 2*lane, 2*lane+1 of the next tile
+    uint64_t start_next[kIn];   // absolute payload offset of the next tile
+    uint64_t start_ctx0[kIn], start_ctx1[kIn];   // of the tiles in the two context buffers (tile parity)
+    auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
+        if constexpr (NIN > 0) {
+            int64_t t = tile_of(r);
+            if (t >= n_tiles) t = 0;   // loads are issued unconditionally; the values are not used then
+#pragma unroll
+            for (int c = 0; c < NIN; ++c) {
+                const uint8_t *h = p.in[c] + (uint64_t)t * kTileBlocks + 2 * lane;
+                hdr_next[c] = (uint32_t)h[0] | ((uint32_t)h[1] << 8);
+                const uint64_t st = p.in_ofs[c][t];
+                start_next[c] = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(st >> 32)) << 32) |
+                                (uint32_t)__builtin_amdgcn_readfirstlane((int)st);
+            }
+        }
+    };
+    // header bytes -> block offsets of tile r in context buffer r & 1 (HomComp/src/GSZ.cu:790-874)
+    auto prepare = [&](int64_t r, int b) __attribute__((always_inline)) {
+        if constexpr (NIN > 0) {
+            if (tile_of(r) < n_tiles) {
+#pragma unroll
+                for (int c = 0; c < NIN; ++c) {
+                    const uint32_t h0 = hdr_next[c] & 0xffu, h1 = hdr_next[c] >> 8;
+                    const uint32_t z0 = size_from_header(h0), z1 = size_from_header(h1);
+                    const uint32_t incl = wave_incl_scan_u32(z0 + z1, lane);
+                    const uint32_t o0 = incl - z0 - z1, o1 = o0 + z0;
+                    *reinterpret_cast<uint32_t *>(&s_ofs_in[wave][c][b][2 * lane]) = o0 | (o1 << 16);
+                    *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)hdr_next[c];
+                    if ((lane & 7) == 0) s_rel[wave][c][b][lane >> 3] = o0;
+                    if (lane == 63) s_rel[wave][c][b][kSub] = incl;
+                    if (b) start_ctx1[c] = start_next[c]; else start_ctx0[c] = start_next[c];
+                }
+                wave_lds_fence();
+            }
+        }
+    };
+
+    // ---- requests kDepth sub-steps ahead, into kDepth register sets used in rotation
+    SubRegs<LOCAL> loc[kDepth];
+    InRegs in[kDepth][kIn];
+    // byte range of sub-step s of the tile in context b: aligned base address, bytes from there
+    auto range_of = [&](int c, int b, int s, uintptr_t &ga, uint32_t &shift, uint32_t &nbytes, uint32_t &rel0)
+                        __attribute__((always_inline)) {
+        rel0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][s]);
+        const uint32_t rel1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][s + 1]);
+        const uint64_t start = b ? start_ctx1[c] : start_ctx0[c];
+        const uint64_t a = start + rel0;
+        uint64_t e = start + rel1;
+        // a block that starts below the stated size is read in full (HomComp/src/GSZ.cu:908-911),
+        // nothing further out is touched
+        const uint64_t lim = p.in_size[c] + (kMaxBlockBytes - 1);
+        if (e > lim) e = lim;
+        const uintptr_t g0 = (uintptr_t)p.in[c] + a;
+        ga = g0 & ~(uintptr_t)15;
+        shift = (uint32_t)(g0 - ga);
+        nbytes = e > a ? shift + (uint32_t)(e - a) : 0u;
+    };
+    // The registers of a set are free again as soon as the sub-step has converted the operand /
+    // staged the chunk, and the request for the sub-step after the next one is issued right there:
+    // as early as possible, and ahead of the sub-step's own stores (a wave's memory operations
+    // complete in order, so a load is only as fast as the stores issued before it).
+    auto request_local = [&](int64_t r, int s, SubRegs<LOCAL> &loc) __attribute__((always_inline)) {
+        const int64_t t = tile_of(r);
+        load_sub<LOCAL>(loc, p.local, p.n, (uint64_t)t * kTileElems, t < n_tiles, s, lane);
+    };
+    auto request_in = [&](int c, int64_t r, int b, int s, InRegs (&in)[kIn]) __attribute__((always_inline)) {
+        uintptr_t ga;
+        uint32_t shift, nbytes, rel0;
+        range_of(c, b, s, ga, shift, nbytes, rel0);
+        // whole 16-byte pieces; lanes beyond the range get zeros without touching memory
+        const __amdgpu_buffer_rsrc_t rs =
+            buffer_of(reinterpret_cast<const void *>(ga), tile_of(r) < n_tiles ? (nbytes + 15u) & ~15u : 0u);
+        in[c].chunk = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 0, kBufNt);
+    };
+    auto request = [&](int64_t r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn]) __attribute__((always_inline)) {
+        request_local(r, s, loc);
+        if constexpr (NIN > 0) {
+#pragma unroll
+            for (int c = 0; c < NIN; ++c) request_in(c, r, b, s, in);
+        }
+    };
+
+    fetch_headers(0);
+    prepare(0, 0);
+#pragma unroll
+    for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j]);
+
+    uint32_t total1 = 0, total2 = 0;   // byte totals of the tiles of the previous two rounds
+    bool spilled1 = false, spilled2 = false;
+    uint64_t probe = 0;                // prefix word of the older one, requested a round ago
+
+    for (int64_t r = 0;; ++r) {
+        const int64_t t0 = tile_of(r), t1 = t0 - GW, t2 = t0 - 2 * GW;
+        const bool v0 = t0 < n_tiles;
+        const bool v1 = kEnc && r >= 1 && t1 < n_tiles;
+        const bool v2 = kEnc && r >= 2 && t2 < n_tiles;
+        if (!v0 && !v1 && !v2) break;
+        const int buf = (int)(r & 1);
+        uint8_t *stage = s_out[wave][buf];
+        uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * 2u + (uint64_t)buf) * kSpillSlotBytes : nullptr;
+
+        // ---- the tile packed two rounds ago goes to its place in the stream
+        if constexpr (kEnc) {
+            if (v2) {
+                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, probe);
+                uint8_t *dst = p.out_cmp + p.hdr_bytes + excl;
+                if (spilled2)
+                    copy_out_spill(slot, dst, total2, lane);
+                else
+                    copy_out<64>(stage, dst, total2, lane);
+            }
+        }
+
+        // ---- this round's tile
+        uint32_t run = 0;
+        bool spilled0 = false;
+        if (v0) {
+            fetch_headers(r + 1);
+            const uint64_t tile_elem0 = (uint64_t)t0 * kTileElems;
+            // sub-step s of this tile; (r2, b2, s2) is the sub-step the freed registers are requested for
+            auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2) __attribute__((always_inline)) {
+                // elements beyond the end arrive as zeros (0.0f quantises to 0), as the reference pads
+                int32_t v[8];
+                if constexpr (LOCAL == kLocalF32) {
+                    // HomComp/src/GSZ.cu:82-149: quantise, Lorenzo with prevQuant = 0 at block start
+                    const float x[8] = {loc.f[0].x, loc.f[0].y, loc.f[0].z, loc.f[0].w,
+                                        loc.f[1].x, loc.f[1].y, loc.f[1].z, loc.f[1].w};
+                    int32_t q[8];
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) q[m] = quantize(x[m], p.recip);
+                    uint32_t prev = dpp_u32<kDppRowShr1>((uint32_t)q[7]);
+                    if (k == 0) prev = 0;
+                    v[0] = (int32_t)((uint32_t)q[0] - prev);
+#pragma unroll
+                    for (int m = 1; m < 8; ++m) v[m] = (int32_t)((uint32_t)q[m] - (uint32_t)q[m - 1]);
+                } else if constexpr (LOCAL == kLocalI32) {
+                    // HomComp/src/homcomp.cu:2252-2268: precomputed deltas
+                    v[0] = loc.i[0].x; v[1] = loc.i[0].y; v[2] = loc.i[0].z; v[3] = loc.i[0].w;
+                    v[4] = loc.i[1].x; v[5] = loc.i[1].y; v[6] = loc.i[1].z; v[7] = loc.i[1].w;
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) v[m] = 0;
+                }
+                request_local(r2, s2, loc);
+                if constexpr (NIN > 0) {
+                    const int blk = s * 16 + quad;
+#pragma unroll
+                    for (int c = 0; c < NIN; ++c) {
+                        // ---- the sub-step's payload range: registers -> LDS stage
+                        uintptr_t ga;
+                        uint32_t shift, nbytes, rel0;
+                        range_of(c, buf, s, ga, shift, nbytes, rel0);
+                        uint8_t *st = s_in[wave][c];
+                        if (16u * (uint32_t)lane < nbytes)
+                            *reinterpret_cast<u32x4 *>(st + 16u * lane) = in[c].chunk;
+                        if (nbytes > 1024u) {   // a range of more than 64 pieces: the rest is fetched now
+                            const __amdgpu_buffer_rsrc_t rs =
+                                buffer_of(reinterpret_cast<const void *>(ga), (nbytes + 15u) & ~15u);
+                            for (uint32_t i = (uint32_t)lane + 64u; 16u * i < nbytes; i += 64u)
+                                *reinterpret_cast<u32x4 *>(st + 16u * i) =
+                                    __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(16u * i), 0, kBufNt);
+                        }
+                        request_in(c, r2, b2, s2, in);
+                        wave_lds_fence();
+                        // ---- decode (HomComp/src/GSZ.cu:883-1434)
+                        const uint32_t h = s_hdr_in[wave][c][buf][blk];
+                        const uint32_t ofs = s_ofs_in[wave][c][buf][blk];
+                        // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
+                        const bool active = size_from_header(h) != 0u && (buf ? start_ctx1[c] : start_ctx0[c]) + ofs < p.in_size[c];
+                        int32_t d[8];
+                        unpack8(st, shift + ofs - rel0, h, active, k, d);
+#pragma unroll
+                        for (int m = 0; m < 8; ++m) v[m] = (int32_t)((uint32_t)v[m] + (uint32_t)d[m]);
+                        wave_lds_fence();   // the stage is rewritten by the next sub-step
+                    }
+                }
+                if constexpr (!kEnc) {
+                    // ---- HomComp/src/GSZ.cu:1426-1468: running sum inside the block, dequantise, store
+                    uint32_t q[8];
+                    q[0] = (uint32_t)v[0];
+#pragma unroll
+                    for (int m = 1; m < 8; ++m) q[m] = q[m - 1] + (uint32_t)v[m];
+                    const uint32_t s0 = dpp_u32<kDppBcast0>(q[7]);
+                    const uint32_t s1 = dpp_u32<kDppBcast1>(q[7]);
+                    const uint32_t s2 = dpp_u32<kDppBcast2>(q[7]);
+                    const uint32_t off = (k > 0 ? s0 : 0u) + (k > 1 ? s1 : 0u) + (k > 2 ? s2 : 0u);
+                    float y[8];
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) y[m] = dequantize((int32_t)(q[m] + off), p.eb);
+                    // The lanes' 32-byte pieces are exchanged through LDS so that each store
+                    // instruction writes 1 KiB of consecutive bytes (full cache lines): stores of
+                    // 16 bytes at a 32-byte stride reach only a fraction of the write bandwidth.
+                    float *tr = s_tr[wave];
+                    *reinterpret_cast<f32x4 *>(tr + 8 * lane) = f32x4{y[0], y[1], y[2], y[3]};
+                    *reinterpret_cast<f32x4 *>(tr + 8 * lane + 4) = f32x4{y[4], y[5], y[6], y[7]};
+                    wave_lds_fence();
+                    const f32x4 lo = *reinterpret_cast<const f32x4 *>(tr + 4 * lane);
+                    const f32x4 hi = *reinterpret_cast<const f32x4 *>(tr + 256 + 4 * lane);
+                    wave_lds_fence();
+                    const __amdgpu_buffer_rsrc_t ro =
+                        buffer_of(p.out_f32 + tile_elem0, tile_elem0 < p.n ? (p.n - tile_elem0) * 4u : 0u);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, lo), ro, lane * 16, s * 2048, kBufNt);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hi), ro, lane * 16 + 1024, s * 2048, kBufNt);
+                } else {
+                    // ---- rate selection (HomComp/src/GSZ.cu:151-167) and the block's offset: the
+                    //      sizes are equal in the four lanes of a quad, so a wave scan of the first
+                    //      lanes' values minus the own size is the exclusive prefix in every lane
+                    uint32_t a[8], sb, hd, size;
+                    analyse8(v, k, a, sb, hd, size);
+                    const uint32_t incl = wave_incl_scan_u32(k == 0 ? size : 0u, lane);
+                    const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+                    const uint32_t pos = run + incl - size;
+                    if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
+                    if (!spilled0 && run + sub_total > (uint32_t)kCap) {
+                        // the tile outgrows the LDS stage: what is packed so far moves to the spill slot
+                        for (uint32_t i = 4u * lane; i < run; i += 256u)
+                            *reinterpret_cast<uint32_t *>(slot + i) = *reinterpret_cast<const uint32_t *>(stage + i);
+                        spilled0 = true;
+                    }
+                    if (spilled0)
+                        pack8((global_bytes)slot, pos, hd, k, a, sb);
+                    else
+                        pack8((lds_bytes)stage, pos, hd, k, a, sb);
+                    run += sub_total;
+                }
+            };
+#pragma unroll 1
+            for (int s = 0; s < kSub; s += kDepth) {
+                // the requests of the last kDepth sub-steps are the next tile's, whose block offsets
+                // must be in place before
+                const int wrap = s + kDepth >= kSub ? 1 : 0;
+                if (wrap) prepare(r + 1, buf ^ 1);
+                const int s2 = s + kDepth - wrap * kSub;
+#pragma unroll
+                for (int j = 0; j < kDepth; ++j) sub(s + j, loc[j], in[j], r + wrap, buf ^ wrap, s2 + j);
+            }
+            if constexpr (kEnc) {
+                wave_lds_fence();
+                // header bytes of the tile (HomComp/src/GSZ.cu:166)
+#pragma unroll
+                for (int i = lane; i < kTileBlocks; i += 64)
+                    p.out_cmp[(uint64_t)t0 * kTileBlocks + i] = s_hdr_out[wave][i];
+                if (lane == 0) scan_publish(scan, (uint32_t)t0, run);
+            }
+        }
+        if constexpr (kEnc) {
+            if (v1) probe = scan_probe(scan, (uint32_t)t1);
+            total2 = total1;
+            total1 = run;
+            spilled2 = spilled1;
+            spilled1 = spilled0;
+        }
     }
 }
 
@@ -686,6 +1089,48 @@ hipError_t tile_kernel_residency(int op, int *blocks_per_cu)
     case kOpHomSumF32: return resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu);
     case kOpHomSumI32: return resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu);
     case kOpHomAdd: return resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int NIN, int LOCAL, int OUT>
+static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_t s)
+{
+    // data workgroups of four waves (one tile per wave and round), on the encoder + the scan server
+    const uint32_t extra = OUT == kOutStream ? 1u : 0u;
+    uint32_t grid = (p.n_tiles + 3u) / 4u + extra;
+    if (grid > max_grid) grid = max_grid;
+    if (grid < 1u + extra) grid = 1u + extra;
+    hipLaunchKernelGGL((k_wave<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), 0, s, p);
+    return hipGetLastError();
+}
+
+template <int NIN, int LOCAL, int OUT>
+static hipError_t wave_resident_blocks(int *blocks_per_cu)
+{
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, 0);
+}
+
+hipError_t wave_kernel_residency(int op, int *blocks_per_cu)
+{
+    switch (op) {
+    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu);
+    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu);
+    case kOpHomSumF32: return wave_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu);
+    case kOpHomSumI32: return wave_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu);
+    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_wave_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
+{
+    switch (op) {
+    case kOpCompress: return launch_wave<0, kLocalF32, kOutStream>(p, max_grid, s);
+    case kOpDecompress: return launch_wave<1, kLocalNone, kOutF32>(p, max_grid, s);
+    case kOpHomSumF32: return launch_wave<1, kLocalF32, kOutStream>(p, max_grid, s);
+    case kOpHomSumI32: return launch_wave<1, kLocalI32, kOutStream>(p, max_grid, s);
+    case kOpHomAdd: return launch_wave<2, kLocalNone, kOutStream>(p, max_grid, s);
     default: return hipErrorInvalidValue;
     }
 }

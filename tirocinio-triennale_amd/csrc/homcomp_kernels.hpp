@@ -38,11 +38,15 @@ struct TileParams {
     uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
     uint64_t *total;            // receives the stream length
     uint64_t *user_total;       // optional second destination for the stream length
+    uint8_t *spill;             // wave kernels: kSpillSlotBytes per data wave and buffer for tiles that outgrow LDS
 };
 
 // Resident workgroups per compute unit for one of the tile kernels (sizes the persistent grid).
 hipError_t tile_kernel_residency(int op, int *blocks_per_cu);
 hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
+hipError_t wave_kernel_residency(int op, int *blocks_per_cu);
+hipError_t launch_wave_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
+constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
 // Tile payload offsets of an incoming stream from its header bytes.
 hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
                              uint32_t *block_sums, uint64_t *ofs, hipStream_t s);
