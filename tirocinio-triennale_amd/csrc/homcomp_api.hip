@@ -51,10 +51,9 @@ struct homcomp_workspace {
     float *d_partial;         // min/max partials
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
-    uint32_t max_grid[hc::kOpCount];  // resident workgroups of each tile kernel on this device
+    uint32_t max_grid[hc::kOpCount];  // workgroups of each operation's kernel that this device keeps resident
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
-    uint32_t wave_grid[hc::kOpCount]; // resident workgroups of each wave kernel (0: none)
-    uint8_t *d_spill;         // spill slots of the wave kernels
+    uint8_t *d_spill;         // spill slots: two worst-case tiles per data wave
 };
 
 namespace {
@@ -108,11 +107,8 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, hipStream_t s)
 {
-    if (ws->wave_grid[op]) {
-        p.spill = ws->d_spill;
-        return hip_ok(hc::launch_wave_op(op, p, ws->wave_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
-    }
-    return hip_ok(hc::launch_tile_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    p.spill = ws->d_spill;
+    return hip_ok(hc::launch_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
 // n == 0: the stream is empty; only the length words are written.
@@ -193,9 +189,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     const size_t bytes = off;
     hipDeviceProp_t prop;
     bool ok = hip_ok(hipGetDeviceProperties(&prop, ws->device));
+    uint32_t widest = 0;
     for (int op = 0; ok && op < hc::kOpCount; ++op) {
         int per_cu = 0;
-        ok = hip_ok(hc::tile_kernel_residency(op, &per_cu));
+        ok = hip_ok(hc::op_kernel_residency(op, &per_cu));
         if (ok && per_cu < 1) per_cu = 1;
         // one compute unit's worth of workgroups is left free: the persistent grid must be fully
         // resident, and an estimate that is off by a single workgroup would stall the launch
@@ -208,30 +205,11 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
             if (pct >= 1 && pct <= 100) ws->max_grid[op] = (uint32_t)((uint64_t)ws->max_grid[op] * (uint64_t)pct / 100u);
         }
         if (ws->max_grid[op] < 2) ws->max_grid[op] = 2;   // an encoder needs a data workgroup and the scan server
-        // decompression has no dependence between tiles: one workgroup per tile, scheduled by the hardware
-        if (op == hc::kOpDecompress) ws->max_grid[op] = 0x7fffffffu;
+        if (op != hc::kOpDecompress && ws->max_grid[op] > widest) widest = ws->max_grid[op];
     }
-    uint32_t max_wave_grid = 0;
-    // Kernel family: the wave-autonomous kernels; HOMCOMP_KERNELS=tile selects the
-    // workgroup-tiled kernels instead (kept for comparisons).
-    const char *family = std::getenv("HOMCOMP_KERNELS");
-    const bool use_wave = !(family && std::strcmp(family, "tile") == 0);
-    for (int op = 0; ok && use_wave && op < hc::kOpCount; ++op) {
-        int per_cu = 0;
-        ok = hip_ok(hc::wave_kernel_residency(op, &per_cu));
-        if (!ok || per_cu < 1) continue;
-        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
-        ws->wave_grid[op] = (uint32_t)per_cu * (uint32_t)cus;
-        if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
-            const long pct = std::strtol(e, nullptr, 10);
-            if (pct >= 1 && pct <= 100) ws->wave_grid[op] = (uint32_t)((uint64_t)ws->wave_grid[op] * (uint64_t)pct / 100u);
-        }
-        if (ws->wave_grid[op] < 2) ws->wave_grid[op] = 2;
-        if (ws->wave_grid[op] > max_wave_grid) max_wave_grid = ws->wave_grid[op];
-    }
-    if (ok && max_wave_grid) {
-        // two slots per data wave, no more waves than tiles
-        size_t waves = (size_t)(max_wave_grid - 1) * 4;
+    if (ok) {
+        // two spill slots per data wave of the widest encoder grid, no more waves than tiles
+        size_t waves = (size_t)(widest > 1 ? widest - 1 : 1) * 4;
         if (waves > ws->max_tiles) waves = ws->max_tiles;
         ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 2 * hc::kSpillSlotBytes));
     }

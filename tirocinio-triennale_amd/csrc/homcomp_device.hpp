@@ -15,18 +15,13 @@
 
 namespace hc {
 
-constexpr int kWG = 256;                              // threads per workgroup (4 waves)
-constexpr int kEPL = 8;                               // elements per lane per iteration
-constexpr int kQuad = 4;                              // lanes per 32-element block
-constexpr int kIter = HC_ITER;                        // iterations per tile
-constexpr int kBlocksPerIter = kWG / kQuad;           // 64
-constexpr int kTileBlocks = kBlocksPerIter * kIter;   // 128
+constexpr int kWG = 256;                              // threads per workgroup (4 independent waves)
+constexpr int kEPL = 8;                               // elements per lane per sub-step
+constexpr int kTileBlocks = 128;                      // blocks per tile
 constexpr int kTileElems = kTileBlocks * 32;          // 4096
 constexpr int kChunkElems = 32768;                    // reference thread-block share
 constexpr int kMaxBlockBytes = 132;                   // largest size a header byte can imply
-constexpr int kStageBytes = kTileBlocks * kMaxBlockBytes + 64;      // LDS stage of an incoming tile
 constexpr int kOutBlockBytes = 128;                   // largest payload the encoder emits per block
-constexpr int kOutStageBytes = kTileBlocks * kOutBlockBytes + 64;   // LDS stage of an outgoing tile
 
 // Native 16-byte vectors (the streaming load/store builtins take these, not HIP's float4).
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -80,20 +75,18 @@ constexpr int kDppRowHalfMirror = 0x141;  // lane i reads lane 7-i inside its gr
 constexpr int kDppRowMirror = 0x140;      // lane i reads lane 15-i inside its row of 16
 
 // Inclusive scan across the wave: Hillis-Steele with DPP row shifts inside each row of 16 lanes,
-// then the totals of the earlier rows through scalar registers.
-// Inclusive scan across the wave: Hillis-Steele with DPP row shifts inside each row of 16 lanes,
-// then the totals of the earlier rows through scalar registers.
-__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int lane)
+// then the row totals travel on with the two row-broadcast steps (lane 15 of a row into the next
+// row, lane 31 into the upper half).  Must run with all lanes active.
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int /*lane*/)
 {
     x += dpp_u32<0x111>(x);   // row_shr:1
     x += dpp_u32<0x112>(x);   // row_shr:2
     x += dpp_u32<0x114>(x);   // row_shr:4
     x += dpp_u32<0x118>(x);   // row_shr:8
-    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)x, 15);
-    const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)x, 31);
-    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)x, 47);
-    const int row = lane >> 4;
-    return x + (row > 0 ? r0 : 0u) + (row > 1 ? r1 : 0u) + (row > 2 ? r2 : 0u);
+    // row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3; other rows keep their value
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xA, 0xF, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xC, 0xF, false);
+    return x;
 }
 
 // ---------------------------------------------------------------- scalar arithmetic
@@ -134,40 +127,49 @@ __device__ __forceinline__ uint32_t size_from_header(uint32_t h)
     return (h & 0x80u) ? 4u + 4u * F + ob : (F ? 4u + 4u * F : 0u);
 }
 
-// Transpose of an 8x8 bit matrix held row-per-byte: result bit (8r+c) = input bit (8c+r).
-__device__ __forceinline__ uint64_t transpose8(uint64_t x)
+// Transpose of an 8x8 bit matrix held row-per-byte in (lo, hi): result bit (8r+c) = input bit
+// (8c+r).  Three rounds of delta swaps; the first two stay inside the 32-bit halves, only the last
+// one moves nibbles between them, so everything is full-rate 32-bit arithmetic.
+__device__ __forceinline__ void transpose8(uint32_t &lo, uint32_t &hi)
 {
-    uint64_t t;
-    t = (x ^ (x >> 7)) & 0x00AA00AA00AA00AAull;
-    x = x ^ t ^ (t << 7);
-    t = (x ^ (x >> 14)) & 0x0000CCCC0000CCCCull;
-    x = x ^ t ^ (t << 14);
-    t = (x ^ (x >> 28)) & 0x00000000F0F0F0F0ull;
-    x = x ^ t ^ (t << 28);
-    return x;
+    uint32_t t;
+    t = (lo ^ (lo >> 7)) & 0x00AA00AAu;
+    lo ^= t ^ (t << 7);
+    t = (hi ^ (hi >> 7)) & 0x00AA00AAu;
+    hi ^= t ^ (t << 7);
+    t = (lo ^ (lo >> 14)) & 0x0000CCCCu;
+    lo ^= t ^ (t << 14);
+    t = (hi ^ (hi >> 14)) & 0x0000CCCCu;
+    hi ^= t ^ (t << 14);
+    // x >> 28 of the 64-bit value, low word only (the mask 0x00000000F0F0F0F0 has no high bits)
+    t = (lo ^ __builtin_amdgcn_alignbit(hi, lo, 28)) & 0xF0F0F0F0u;
+    lo ^= t ^ (t << 28);
+    hi ^= t >> 4;
 }
 
 // ---------------------------------------------------------------- per-lane block pieces
 
 // Encoder front end for one lane's 8 signed deltas (HomComp/src/GSZ.cu:86-164): sign byte,
 // magnitudes, block-wide bit widths through the quad, rate selection.  `k` is the lane's
-// position in its quad.  hdr and size come out identical in the four lanes of a quad.
+// position in its quad.  hdr, size and a0 (|delta| of the block's element 0) come out identical
+// in the four lanes of a quad.
 __device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8], uint32_t &sb,
-                                         uint32_t &hdr, uint32_t &size)
+                                         uint32_t &hdr, uint32_t &size, uint32_t &a0)
 {
     sb = 0;
     uint32_t rest = 0;
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
-        uint32_t neg = v[m] < 0 ? 1u : 0u;
-        a[m] = neg ? 0u - (uint32_t)v[m] : (uint32_t)v[m];
-        sb |= neg << (7 - m);
+        const uint32_t u = (uint32_t)v[m];
+        const int32_t neg = (int32_t)(0u - u);
+        a[m] = (uint32_t)(v[m] > neg ? v[m] : neg);        // |v| (0x80000000 stays, as in the reference)
+        sb = __builtin_amdgcn_alignbit(sb, u, 31);        // shift in the sign bit: element 0 ends at bit 7
         if (m) rest |= a[m];
     }
     // bit width of a maximum equals the bit width of the OR
     uint32_t or1 = quad_or(rest | a[0]);                  // all 32 elements   (:152)
     uint32_t or2 = quad_or(rest | (k ? a[0] : 0u));       // elements 1..31    (:153)
-    uint32_t a0 = dpp_u32<kDppBcast0>(a[0]);              // element 0         (:154)
+    a0 = dpp_u32<kDppBcast0>(a[0]);                       // element 0         (:154)
     uint32_t fr1 = planes_of(or1);
     uint32_t fr2 = planes_of(or2);
     uint32_t ob = (bit_num(a0) + 7u) >> 3;
@@ -183,97 +185,106 @@ __device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8
 }
 
 // Encoder back end for one lane (HomComp/src/GSZ.cu:245-751): writes this lane's share of the
-// block payload into the LDS stage at `pos0` (the block's tile-relative offset).  Lane k
-// contributes byte k of the sign word and of every plane; lane 0 also writes the outlier bytes.
+// block payload into the stage at `pos0` (the block's tile-relative offset).  Lane k contributes
+// byte k of the sign word and of every plane, and byte k of the outlier.
+//
+// The code is kept free of per-plane branches: planes are written in whole groups of eight, so a
+// lane also stores bytes for planes its block does not have.  Those land in the space of the
+// blocks that follow (at most 35 bytes past the block's end) and are harmless because of the
+// store order: planes from the highest to the lowest, then the sign bytes, then the outlier bytes.
+// If a stray byte of block B and a valid plane byte of a later block X fall on one address, X's
+// plane index is lower (X starts at least 4 bytes after B's first plane), so X's store is issued
+// later and wins; sign and outlier bytes are issued after all plane stores.  Blocks without
+// payload must not store at all (they share their position with the next block).  The stages
+// keep 64 bytes of slack behind the last block.
+//
 // `stage` may carry an explicit address space (lds_bytes / global_bytes below) so that two calls
 // with different destinations cannot be merged into one sequence of flat stores.
 typedef __attribute__((address_space(3))) uint8_t *lds_bytes;
 typedef __attribute__((address_space(1))) uint8_t *global_bytes;
 
+template <int G, typename Bytes>
+__device__ __forceinline__ void pack_group(Bytes stage, uint32_t base, const uint32_t a[8])
+{
+    // byte r of (lo, hi) = bits 8G..8G+7 of a[7-r]; after the transpose byte r is plane 8G+r
+    constexpr uint32_t two = 0x0c0c0400u + 0x0101u * (uint32_t)G;   // byte G of the second, then of the first operand
+    uint32_t lo = __builtin_amdgcn_perm(__builtin_amdgcn_perm(a[4], a[5], two),
+                                        __builtin_amdgcn_perm(a[6], a[7], two), 0x05040100u);
+    uint32_t hi = __builtin_amdgcn_perm(__builtin_amdgcn_perm(a[0], a[1], two),
+                                        __builtin_amdgcn_perm(a[2], a[3], two), 0x05040100u);
+    transpose8(lo, hi);
+#pragma unroll
+    for (int r = 7; r >= 0; --r)
+        stage[base + 4u * (uint32_t)(8 * G + r)] = (uint8_t)((r < 4 ? lo : hi) >> (8 * (r & 3)));
+}
+
 template <typename Bytes>
 __device__ __forceinline__ void pack8(Bytes stage, uint32_t pos0, uint32_t hdr, int k,
-                                      uint32_t a[8], uint32_t sb)
+                                      const uint32_t a_in[8], uint32_t sb, uint32_t a0)
 {
+    if (hdr == 0) return;                                 // zero block (:287)
     const uint32_t sel = hdr >> 7;
     const uint32_t F = hdr & 0x1fu;
-    if (!sel && F == 0) return;                           // zero block (:287)
-    uint32_t pos = pos0;
-    if (sel) {
-        const uint32_t ob = ((hdr >> 5) & 3u) + 1u;
-        if (k == 0) {
-            uint32_t a0 = a[0];
-            for (uint32_t i = 0; i < ob; ++i) {           // little-endian outlier (:271-275)
-                stage[pos0 + i] = (uint8_t)a0;
-                a0 >>= 8;
-            }
-            a[0] = 0;                                     // element 0 leaves the planes (:274)
-        }
-        pos += ob;
-    }
-    stage[pos + k] = (uint8_t)sb;                         // sign word, MSB = element 0 (:292-295)
-    pos += 4 + k;
-    const uint32_t groups = (F + 7u) >> 3;
+    const uint32_t ob = sel ? ((hdr >> 5) & 3u) + 1u : 0u;
+    uint32_t a[8];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        if ((uint32_t)g < groups) {
-            // byte r of x = bits 8g..8g+7 of a[7-r]; after the transpose byte r is plane 8g+r
-            uint32_t lo = ((a[7] >> (8 * g)) & 0xffu) | (((a[6] >> (8 * g)) & 0xffu) << 8) |
-                          (((a[5] >> (8 * g)) & 0xffu) << 16) | (((a[4] >> (8 * g)) & 0xffu) << 24);
-            uint32_t hi = ((a[3] >> (8 * g)) & 0xffu) | (((a[2] >> (8 * g)) & 0xffu) << 8) |
-                          (((a[1] >> (8 * g)) & 0xffu) << 16) | (((a[0] >> (8 * g)) & 0xffu) << 24);
-            uint64_t y = transpose8(((uint64_t)hi << 32) | lo);
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                if ((uint32_t)(8 * g + r) < F)
-                    stage[pos + 4u * (uint32_t)(8 * g + r)] = (uint8_t)(y >> (8 * r));
-            }
-        }
-    }
+    for (int m = 1; m < 8; ++m) a[m] = a_in[m];
+    a[0] = (sel && k == 0) ? 0u : a_in[0];                // element 0 leaves the planes (:274)
+    const uint32_t base = pos0 + ob + 4u + (uint32_t)k;
+    if (F > 24u) pack_group<3>(stage, base, a);
+    if (F > 16u) pack_group<2>(stage, base, a);
+    if (F > 8u) pack_group<1>(stage, base, a);
+    pack_group<0>(stage, base, a);
+    stage[pos0 + ob + (uint32_t)k] = (uint8_t)sb;         // sign word, MSB = element 0 (:292-295)
+    if ((uint32_t)k < ob) stage[pos0 + (uint32_t)k] = (uint8_t)(a0 >> (8 * k));   // little-endian outlier (:271-275)
 }
 
 // Decoder for one lane (HomComp/src/GSZ.cu:883-1434 up to the signed deltas): reads this lane's
 // bytes of the block payload at `pos0` in the LDS stage.  Inactive blocks (rate 0, or payload
-// offset beyond the stated stream size, :908-911) give zero deltas.
+// offset beyond the stated stream size, :908-911) give zero deltas.  Branch-free like pack8: the
+// first eight plane bytes are always read (up to 35 bytes past the block's end, inside the
+// stage's slack) and the planes the block does not have are cut off when the bits are extracted.
+// Must run with all lanes of the wave active (the outlier bytes are gathered across the quad).
+template <int G>
+__device__ __forceinline__ void unpack_group(const uint8_t *stage, uint32_t base, uint32_t width, uint32_t a[8])
+{
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const uint32_t byte = stage[base + 4u * (uint32_t)(8 * G + r)];
+        if (r < 4) lo |= byte << (8 * r); else hi |= byte << (8 * (r - 4));
+    }
+    transpose8(lo, hi);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        // byte r = the block's planes 8G..8G+7 of element 7-r; only `width` of them exist
+        const uint32_t bits = __builtin_amdgcn_ubfe(r < 4 ? lo : hi, 8 * (r & 3), width);
+        a[7 - r] = G == 0 ? bits : a[7 - r] | (bits << (8 * G));
+    }
+}
+
 __device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uint32_t hdr,
                                         bool active, int k, int32_t v[8])
 {
+    if (!active) hdr = 0;
+    const uint32_t sel = hdr >> 7;
+    const uint32_t F = hdr & 0x1fu;
+    const uint32_t ob = sel ? ((hdr >> 5) & 3u) + 1u : 0u;
+    const uint32_t base = pos0 + ob + 4u + (uint32_t)k;
     uint32_t a[8];
-#pragma unroll
-    for (int m = 0; m < 8; ++m) a[m] = 0;
-    uint32_t sb = 0;
-    if (active) {
-        const uint32_t sel = hdr >> 7;
-        const uint32_t F = hdr & 0x1fu;
-        const uint32_t ob = sel ? ((hdr >> 5) & 3u) + 1u : 0u;
-        uint32_t pos = pos0 + ob;
-        sb = stage[pos + k];                              // :921-924, :990-994
-        pos += 4 + k;
-        const uint32_t groups = (F + 7u) >> 3;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            if ((uint32_t)g < groups) {
-                uint64_t y = 0;
-#pragma unroll
-                for (int r = 0; r < 8; ++r) {
-                    if ((uint32_t)(8 * g + r) < F)
-                        y |= (uint64_t)stage[pos + 4u * (uint32_t)(8 * g + r)] << (8 * r);
-                }
-                uint64_t x = transpose8(y);
-#pragma unroll
-                for (int r = 0; r < 8; ++r)
-                    a[7 - r] |= (uint32_t)((x >> (8 * r)) & 0xffu) << (8 * g);
-            }
-        }
-        if (sel && k == 0) {                              // :913-917, :986-987, :1005-1006
-            uint32_t o = 0;
-            for (uint32_t i = 0; i < ob; ++i) o |= (uint32_t)stage[pos0 + i] << (8 * i);
-            a[0] = o;
-        }
-    }
+    unpack_group<0>(stage, base, F < 8u ? F : 8u, a);
+    if (F > 8u) unpack_group<1>(stage, base, F < 16u ? F - 8u : 8u, a);
+    if (F > 16u) unpack_group<2>(stage, base, F < 24u ? F - 16u : 8u, a);
+    if (F > 24u) unpack_group<3>(stage, base, F - 24u, a);
+    const uint32_t sb = hdr ? stage[pos0 + ob + (uint32_t)k] : 0u;   // :921-924, :990-994
+    // outlier: lane k reads byte k, the quad ORs the pieces together (:913-917, :986-987, :1005-1006)
+    const uint32_t piece = (uint32_t)k < ob ? (uint32_t)stage[pos0 + (uint32_t)k] << (8 * k) : 0u;
+    const uint32_t o = quad_or(piece);
+    if (sel && k == 0) a[0] = o;
 #pragma unroll
     for (int m = 0; m < 8; ++m) {                         // :1432-1434
-        uint32_t neg = (sb >> (7 - m)) & 1u;
-        v[m] = (int32_t)(neg ? 0u - a[m] : a[m]);
+        const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)sb, 7 - m, 1);   // 0 or ~0
+        v[m] = (int32_t)((a[m] ^ mask) - mask);
     }
 }
 

@@ -1,101 +1,29 @@
 // HomComp kernels for gfx950.
 //
-// k_tile<NIN, LOCAL, OUT> is one persistent, tiled, single-pass kernel template that covers
-// compress, decompress and the three homomorphic sums.  A tile is 4096 elements = 128 blocks,
-// processed by one 256-thread workgroup in two iterations of 8 elements per lane.  The grid is
-// sized to what the device can keep resident and walks the tiles in rounds
-// (tile = blockIdx.x, += gridDim.x), so the loads of the next tile are issued while the
-// current one is still being packed and stored.  Phases per tile:
-//   1. local operand (float32 values or int32 deltas) -> registers (prefetched one tile ahead)
-//   2. per incoming stream: tile payload offset from the offsets array that k_in_totals /
-//      k_in_scan produced from the header bytes; header bytes -> block sizes -> tile-local
-//      scan; coalesced 16-byte copy of the payload into LDS; per-lane decode
-//   3. combine: delta_out = delta_local + decoded deltas (HomComp/src/homcomp.cu:3611-3616)
-//   4a. stream output: rate selection, header bytes, tile-local scan, pack into one of two LDS
-//       buffers; the tile's offset in the stream comes from the scan-server workgroup of the
-//       same launch (publish the tile total in this round, request the prefix in the next, use
-//       it in the one after), so the payload is copied to the stream (coalesced 16-byte stores)
-//       two rounds after it was packed and no data workgroup waits for another
-//   4b. float output: in-block running sum, dequantise, two float4 stores per lane
-// Small streaming kernels cover the incoming-stream offsets, the Lorenzo pre-pass and the
-// value range.
+// k_wave<NIN, LOCAL, OUT> is one persistent, single-pass kernel template that covers compress,
+// decompress and the three homomorphic sums (NIN incoming streams, a local operand of float32
+// values / int32 deltas / nothing, stream or float32 output).  A tile is 4096 elements = 128
+// blocks and belongs to one wave; the scan-server workgroup of the same launch turns the tiles'
+// byte totals into their offsets in the outgoing stream.  Small streaming kernels cover the
+// incoming-stream offsets, the Lorenzo pre-pass and the value range.
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
+#ifndef HC_CAP0
+#define HC_CAP0 4096
+#endif
+#ifndef HC_CAP1
+#define HC_CAP1 3072
+#endif
+#ifndef HC_DEPTH_ENC
+#define HC_DEPTH_ENC 2
+#endif
 namespace hc {
-
-// Tile-local exclusive scan of the block sizes of a tile, run by one wave; returns the tile
-// total in every lane.
-__device__ __forceinline__ uint32_t tile_scan(const uint32_t *s_size, uint32_t *s_ofs, int lane)
-{
-    constexpr int kPer = kTileBlocks / 64;   // blocks per lane
-    uint32_t sz[kPer], sum = 0;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        sz[j] = s_size[kPer * lane + j];
-        sum += sz[j];
-    }
-    const uint32_t incl = wave_incl_scan_u32(sum, lane);
-    uint32_t run = incl - sum;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        s_ofs[kPer * lane + j] = run;
-        run += sz[j];
-    }
-    return (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-}
-
-// Registers holding one tile's share of the local operand.
-template <int LOCAL>
-struct LocalRegs {
-    f32x4 f[kIter][2];
-    i32x4 i[kIter][2];
-};
-
-template <int LOCAL>
-__device__ __forceinline__ void load_local(LocalRegs<LOCAL> &r, const void *local, uint64_t n,
-                                           uint64_t tile_elem0, int tid)
-{
-    if constexpr (LOCAL == kLocalNone) return;
-#pragma unroll
-    for (int it = 0; it < kIter; ++it) {
-        const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
-        if (e0 + kEPL <= n) {
-            if constexpr (LOCAL == kLocalF32) {
-                const float *src = (const float *)local + e0;
-                r.f[it][0] = stream_load<f32x4>(src);
-                r.f[it][1] = stream_load<f32x4>(src + 4);
-            } else {
-                const int32_t *src = (const int32_t *)local + e0;
-                r.i[it][0] = stream_load<i32x4>(src);
-                r.i[it][1] = stream_load<i32x4>(src + 4);
-            }
-        } else {
-            float tf[8];
-            int32_t ti[8];
-#pragma unroll
-            for (int m = 0; m < 8; ++m) {
-                const bool in = e0 + m < n;
-                if constexpr (LOCAL == kLocalF32)
-                    tf[m] = in ? ((const float *)local)[e0 + m] : 0.0f;
-                else
-                    ti[m] = in ? ((const int32_t *)local)[e0 + m] : 0;
-            }
-            if constexpr (LOCAL == kLocalF32) {
-                r.f[it][0] = f32x4{tf[0], tf[1], tf[2], tf[3]};
-                r.f[it][1] = f32x4{tf[4], tf[5], tf[6], tf[7]};
-            } else {
-                r.i[it][0] = i32x4{ti[0], ti[1], ti[2], ti[3]};
-                r.i[it][1] = i32x4{ti[4], ti[5], ti[6], ti[7]};
-            }
-        }
-    }
-}
 
 // Coalesced copy of a packed tile payload from LDS to its (arbitrarily aligned) place in the
 // stream: bytes up to the first 16-byte boundary, aligned 16-byte stores assembled from
 // unaligned LDS words with v_alignbyte, then the remaining bytes.
-template <int LANES = kWG>
+template <int LANES>
 __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint32_t tot, int tid)
 {
     const uint32_t mis = (uint32_t)((uintptr_t)g & 15u);
@@ -119,9 +47,6 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
     }
     if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = stage[head + 16u * nch + tid];
 }
-
-template <int OUT>
-constexpr int tile_threads() { return kWG; }
 
 // The scan server: one workgroup of the launch that turns the tile totals the data workgroups
 // publish into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  It sweeps the tiles in index
@@ -219,239 +144,6 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
     }
 }
 
-template <int NIN, int LOCAL, int OUT>
-__global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p)
-{
-    constexpr bool kEnc = OUT == kOutStream;
-    constexpr int kLead = tile_threads<OUT>() - kWG;
-    constexpr int kIn = NIN > 0 ? NIN : 1;
-    __shared__ __align__(16) uint8_t s_in[kIn][NIN > 0 ? kStageBytes : 16];
-    __shared__ __align__(16) uint8_t s_out[2][kEnc ? kOutStageBytes : 16];
-    __shared__ uint32_t s_size[kTileBlocks];
-    __shared__ uint32_t s_ofs_in[kIn][kTileBlocks];
-    __shared__ uint32_t s_ofs_out[kTileBlocks];
-    __shared__ uint8_t s_hdr_in[kIn][kTileBlocks];
-    __shared__ uint8_t s_hdr_out[kTileBlocks];
-    __shared__ uint64_t s_base;
-    __shared__ uint32_t s_total;
-
-    const int tid = (int)threadIdx.x - kLead;   // data lane index, negative in the scan wave
-    const bool data = tid >= 0;                 // wave-uniform
-    const bool scanw = threadIdx.x < 64;        // the wave that runs tile-local and global scans
-    const int lane = threadIdx.x & 63;
-    const int k = tid & 3;
-    const int quad = tid >> 2;
-    const int64_t n_tiles = p.n_tiles;
-    const ScanCtx scan{p.tile_totals, p.tile_prefixes, p.n_tiles, p.epoch, p.spin_limit, p.error};
-    // on the encoder the last workgroup of the grid is the scan server, the others walk the tiles
-    const int64_t G = kEnc ? (int64_t)gridDim.x - 1 : (int64_t)gridDim.x;
-    if constexpr (kEnc) {
-        if ((int64_t)blockIdx.x == G) {
-            scan_server(p, scan, (uint32_t)G);
-            return;
-        }
-    }
-
-    // The local operand is prefetched two rounds ahead into two register sets that the rounds
-    // use alternately.  A wave's memory operations complete in issue order and s_waitcnt can only
-    // wait for "all but the N youngest", so a load must never be waited for while younger bulk
-    // loads are still in flight: every load here is at least one full round old when it is used.
-    LocalRegs<LOCAL> buf_a, buf_b;
-    if (data && (int64_t)blockIdx.x < n_tiles)
-        load_local<LOCAL>(buf_a, p.local, p.n, (uint64_t)blockIdx.x * kTileElems, tid);
-    if (data && (int64_t)blockIdx.x + G < n_tiles)
-        load_local<LOCAL>(buf_b, p.local, p.n, (uint64_t)(blockIdx.x + G) * kTileElems, tid);
-
-    // scan pipeline registers of wave 0: byte totals of the tiles of the previous two rounds and
-    // the prefix word requested in the previous round for the older of the two
-    uint32_t total1 = 0, total2 = 0;
-    uint64_t probe = 0;
-
-    // A round handles tile t0 (operand in `nxt`) and, on the encoder, finishes the scan and the
-    // store of the tiles of the two rounds before (t1, t2).  Returns false when nothing is left.
-    auto round = [&](const int64_t t0, LocalRegs<LOCAL> &nxt) __attribute__((always_inline)) -> bool {
-        const int64_t t1 = t0 - G, t2 = t0 - 2 * G;
-        const bool v0 = t0 < n_tiles;
-        const bool v1 = kEnc && t1 >= 0 && t1 < n_tiles;
-        const bool v2 = kEnc && t2 >= 0 && t2 < n_tiles;
-        if (!v0 && !v1 && !v2) return false;
-        const uint32_t tile = (uint32_t)t0;
-        const int buf = (int)((t0 / G) & 1);
-
-        uint32_t a[kIter][8], sb[kIter], hd[kIter];
-        if (v0) {
-            const uint64_t tile_elem0 = (uint64_t)tile * kTileElems;
-
-            // ---- incoming streams: header bytes, block offsets, payload into LDS
-            uint64_t in_base[kIn];
-            uint32_t in_shift[kIn];
-#pragma unroll
-            for (int c = 0; c < NIN; ++c) {
-                const uint64_t start = p.in_ofs[c][tile];
-                const uint32_t total = (uint32_t)(p.in_ofs[c][tile + 1] - start);
-                in_base[c] = start;
-                if (data && tid < kTileBlocks) {
-                    const uint32_t h = p.in[c][(uint64_t)tile * kTileBlocks + tid];
-                    s_hdr_in[c][tid] = (uint8_t)h;
-                    s_size[tid] = size_from_header(h);
-                }
-                const uintptr_t g0 = (uintptr_t)p.in[c] + start;
-                const uintptr_t ga = g0 & ~(uintptr_t)15;
-                const uint32_t shift = (uint32_t)(g0 - ga);
-                in_shift[c] = shift;
-                const uint32_t nbytes = total ? shift + total : 0u;
-                const uint32_t nchunks = data ? (nbytes + 15u) >> 4 : 0u;
-                for (uint32_t i = (uint32_t)tid; i < nchunks; i += kWG) {
-                    if (16u * (i + 1u) <= nbytes) {
-                        *reinterpret_cast<u32x4 *>(&s_in[c][16u * i]) =
-                            stream_load_global<u32x4>(ga + 16u * (uintptr_t)i);
-                    } else {
-                        for (uint32_t j = 16u * i; j < nbytes; ++j)
-                            s_in[c][j] = *reinterpret_cast<const uint8_t *>(ga + j);
-                    }
-                }
-                __syncthreads();
-                if (scanw) tile_scan(s_size, s_ofs_in[c], lane);
-                __syncthreads();
-            }
-
-            if (data) {
-            // ---- per iteration: local deltas + decoded deltas
-            int32_t v[kIter][8];
-#pragma unroll
-            for (int it = 0; it < kIter; ++it) {
-                const int blk = it * kBlocksPerIter + quad;
-                if constexpr (LOCAL == kLocalF32) {
-                    // HomComp/src/GSZ.cu:82-149: quantise, Lorenzo with prevQuant = 0 at block start
-                    const float x[8] = {nxt.f[it][0].x, nxt.f[it][0].y, nxt.f[it][0].z, nxt.f[it][0].w,
-                                        nxt.f[it][1].x, nxt.f[it][1].y, nxt.f[it][1].z, nxt.f[it][1].w};
-                    int32_t q[8];
-#pragma unroll
-                    for (int m = 0; m < 8; ++m) q[m] = quantize(x[m], p.recip);
-                    uint32_t prev = dpp_u32<kDppRowShr1>((uint32_t)q[7]);
-                    if (k == 0) prev = 0;
-                    v[it][0] = (int32_t)((uint32_t)q[0] - prev);
-#pragma unroll
-                    for (int m = 1; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)q[m] - (uint32_t)q[m - 1]);
-                } else if constexpr (LOCAL == kLocalI32) {
-                    // HomComp/src/homcomp.cu:2252-2268: precomputed deltas
-                    v[it][0] = nxt.i[it][0].x; v[it][1] = nxt.i[it][0].y; v[it][2] = nxt.i[it][0].z; v[it][3] = nxt.i[it][0].w;
-                    v[it][4] = nxt.i[it][1].x; v[it][5] = nxt.i[it][1].y; v[it][6] = nxt.i[it][1].z; v[it][7] = nxt.i[it][1].w;
-                } else {
-#pragma unroll
-                    for (int m = 0; m < 8; ++m) v[it][m] = 0;
-                }
-#pragma unroll
-                for (int c = 0; c < NIN; ++c) {
-                    const uint32_t h = s_hdr_in[c][blk];
-                    const uint32_t ofs = s_ofs_in[c][blk];
-                    // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
-                    const bool active = size_from_header(h) != 0u && in_base[c] + ofs < p.in_size[c];
-                    int32_t d[8];
-                    unpack8(s_in[c], in_shift[c] + ofs, h, active, k, d);
-#pragma unroll
-                    for (int m = 0; m < 8; ++m) v[it][m] = (int32_t)((uint32_t)v[it][m] + (uint32_t)d[m]);
-                }
-            }
-
-            if constexpr (!kEnc) {
-                // ---- the operand of the round after the next one starts to fly now
-                if (t0 + 2 * G < n_tiles)
-                    load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
-                // ---- HomComp/src/GSZ.cu:1426-1468: running sum inside the block, dequantise, store
-#pragma unroll
-                for (int it = 0; it < kIter; ++it) {
-                    uint32_t q[8];
-                    q[0] = (uint32_t)v[it][0];
-#pragma unroll
-                    for (int m = 1; m < 8; ++m) q[m] = q[m - 1] + (uint32_t)v[it][m];
-                    const uint32_t s0 = dpp_u32<kDppBcast0>(q[7]);
-                    const uint32_t s1 = dpp_u32<kDppBcast1>(q[7]);
-                    const uint32_t s2 = dpp_u32<kDppBcast2>(q[7]);
-                    const uint32_t off = (k > 0 ? s0 : 0u) + (k > 1 ? s1 : 0u) + (k > 2 ? s2 : 0u);
-                    float y[8];
-#pragma unroll
-                    for (int m = 0; m < 8; ++m) y[m] = dequantize((int32_t)(q[m] + off), p.eb);
-                    const uint64_t e0 = tile_elem0 + (uint64_t)it * (kWG * kEPL) + (uint64_t)tid * kEPL;
-                    if (e0 + kEPL <= p.n) {
-                        float *dst = p.out_f32 + e0;
-                        stream_store<f32x4>(dst, f32x4{y[0], y[1], y[2], y[3]});
-                        stream_store<f32x4>(dst + 4, f32x4{y[4], y[5], y[6], y[7]});
-                    } else {
-#pragma unroll
-                        for (int m = 0; m < 8; ++m)
-                            if (e0 + m < p.n) p.out_f32[e0 + m] = y[m];
-                    }
-                }
-            } else {
-                // ---- rate selection and header bytes (HomComp/src/GSZ.cu:151-167)
-#pragma unroll
-                for (int it = 0; it < kIter; ++it) {
-                    uint32_t size;
-                    analyse8(v[it], k, a[it], sb[it], hd[it], size);
-                    if (k == 0) {
-                        const int blk = it * kBlocksPerIter + quad;
-                        s_size[blk] = size;
-                        s_hdr_out[blk] = (uint8_t)hd[it];
-                    }
-                }
-            }
-            }  // data
-            if constexpr (!kEnc) __syncthreads();  // LDS of this tile is dead before the next round overwrites it
-        }
-
-        if constexpr (kEnc) {
-            // ---- wave 0 runs the scan steps (HomComp/src/GSZ.cu:170-239).  A wave's memory
-            //      operations complete in issue order, so the resolve step, which needs the probe
-            //      issued a round ago, comes before this round's stores and loads of the wave.
-            if (scanw && v2) {
-                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, probe);
-                if (lane == 0) {
-                    s_base = p.hdr_bytes + excl;
-                    s_total = total2;
-                }
-            }
-            __syncthreads();
-            if (scanw) {
-                uint32_t total0 = 0;
-                if (v0) {
-                    total0 = tile_scan(s_size, s_ofs_out, lane);
-                    if (lane == 0) scan_publish(scan, tile, total0);
-                }
-                if (v1) probe = scan_probe(scan, (uint32_t)t1);
-                total2 = total1;
-                total1 = total0;
-            }
-            if (v0 && data && tid < kTileBlocks) p.out_cmp[(uint64_t)tile * kTileBlocks + tid] = s_hdr_out[tid];
-            // ---- the tile packed two rounds ago goes to its place in the stream
-            if (v2 && data) {
-                const uint64_t gofs = s_base;
-                const uint32_t tot = s_total;
-                copy_out(s_out[buf], p.out_cmp + gofs, tot, tid);
-            }
-            __syncthreads();
-            // ---- the operand of the round after the next one starts to fly now
-            if (data && t0 + 2 * G < n_tiles)
-                load_local<LOCAL>(nxt, p.local, p.n, (uint64_t)(t0 + 2 * G) * kTileElems, tid);
-            // ---- and this round's tile takes over the buffer (HomComp/src/GSZ.cu:241-751)
-            if (v0 && data) {
-#pragma unroll
-                for (int it = 0; it < kIter; ++it) {
-                    const int blk = it * kBlocksPerIter + quad;
-                    pack8(s_out[buf], s_ofs_out[blk], hd[it], k, a[it], sb[it]);
-                }
-            }
-        }
-        return true;
-    };
-
-    for (int64_t t0 = blockIdx.x;; t0 += 2 * G) {
-        if (!round(t0, buf_a)) break;
-        if (!round(t0 + G, buf_b)) break;
-    }
-}
-
-
 // ---------------------------------------------------------------- wave-autonomous kernels
 //
 // k_wave<NIN, LOCAL, OUT>: all five operations with one tile per WAVE and no workgroup barrier
@@ -475,10 +167,10 @@ __global__ __launch_bounds__(tile_threads<OUT>()) void k_tile(const TileParams p
 // wave_cap() bytes (the budget that lets 12-16 waves share a compute unit); a tile that outgrows
 // it continues in the wave's slot of a global spill area and is copied out from there.
 constexpr int kSub = kTileBlocks / 16;
-constexpr int kInStage = 16 * kMaxBlockBytes + 48;   // one sub-step's payload range plus alignment slack
+constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
 
 template <int NIN>
-constexpr int wave_cap() { return NIN == 0 ? 4096 : (NIN == 1 ? 3072 : 2048); }
+constexpr int wave_cap() { return NIN == 0 ? HC_CAP0 : (NIN == 1 ? HC_CAP1 : 2048); }
 
 template <int LOCAL>
 struct SubRegs {
@@ -566,7 +258,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // Sub-steps between a request and its use.  A wave's memory operations complete in order, so
     // waiting for a load also waits for every store issued before it: the decoder, which stores
     // 2 KiB per sub-step, looks further ahead to keep more of its stores in flight.
-    constexpr int kDepth = kEnc ? 2 : 4;
+    constexpr int kDepth = HC_DEPTH_ENC > 0 && kEnc ? HC_DEPTH_ENC : 4;
     static_assert(kSub % kDepth == 0, "the register sets rotate with the sub-steps of a tile");
     __shared__ __align__(16) uint8_t s_out[kW][2][kEnc ? kCap + 64 : 16];
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
@@ -805,8 +497,8 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     // ---- rate selection (HomComp/src/GSZ.cu:151-167) and the block's offset: the
                     //      sizes are equal in the four lanes of a quad, so a wave scan of the first
                     //      lanes' values minus the own size is the exclusive prefix in every lane
-                    uint32_t a[8], sb, hd, size;
-                    analyse8(v, k, a, sb, hd, size);
+                    uint32_t a[8], sb, hd, size, a0;
+                    analyse8(v, k, a, sb, hd, size, a0);
                     const uint32_t incl = wave_incl_scan_u32(k == 0 ? size : 0u, lane);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     const uint32_t pos = run + incl - size;
@@ -818,9 +510,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         spilled0 = true;
                     }
                     if (spilled0)
-                        pack8((global_bytes)slot, pos, hd, k, a, sb);
+                        pack8((global_bytes)slot, pos, hd, k, a, sb, a0);
                     else
-                        pack8((lds_bytes)stage, pos, hd, k, a, sb);
+                        pack8((lds_bytes)stage, pos, hd, k, a, sb, a0);
                     run += sub_total;
                 }
             };
@@ -1063,37 +755,6 @@ __global__ void k_fill_u64(uint64_t *p, uint64_t n)
 // ---------------------------------------------------------------- launchers
 
 template <int NIN, int LOCAL, int OUT>
-static hipError_t launch_tile(const TileParams &p, uint32_t max_grid, hipStream_t s)
-{
-    // encoder: data workgroups + the scan server, together no more than the device keeps resident
-    const uint32_t extra = OUT == kOutStream ? 1u : 0u;
-    uint32_t grid = p.n_tiles + extra;
-    if (grid > max_grid) grid = max_grid;
-    if (grid < 1u + extra) grid = 1u + extra;
-    hipLaunchKernelGGL((k_tile<NIN, LOCAL, OUT>), dim3(grid), dim3(tile_threads<OUT>()), 0, s, p);
-    return hipGetLastError();
-}
-
-template <int NIN, int LOCAL, int OUT>
-static hipError_t resident_blocks(int *blocks_per_cu)
-{
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_tile<NIN, LOCAL, OUT>,
-                                                        tile_threads<OUT>(), 0);
-}
-
-hipError_t tile_kernel_residency(int op, int *blocks_per_cu)
-{
-    switch (op) {
-    case kOpCompress: return resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu);
-    case kOpDecompress: return resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu);
-    case kOpHomSumF32: return resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu);
-    case kOpHomSumI32: return resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu);
-    case kOpHomAdd: return resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu);
-    default: return hipErrorInvalidValue;
-    }
-}
-
-template <int NIN, int LOCAL, int OUT>
 static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     // data workgroups of four waves (one tile per wave and round), on the encoder + the scan server
@@ -1111,7 +772,7 @@ static hipError_t wave_resident_blocks(int *blocks_per_cu)
     return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, 0);
 }
 
-hipError_t wave_kernel_residency(int op, int *blocks_per_cu)
+hipError_t op_kernel_residency(int op, int *blocks_per_cu)
 {
     switch (op) {
     case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu);
@@ -1123,7 +784,7 @@ hipError_t wave_kernel_residency(int op, int *blocks_per_cu)
     }
 }
 
-hipError_t launch_wave_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
+hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     switch (op) {
     case kOpCompress: return launch_wave<0, kLocalF32, kOutStream>(p, max_grid, s);
@@ -1131,18 +792,6 @@ hipError_t launch_wave_op(int op, const TileParams &p, uint32_t max_grid, hipStr
     case kOpHomSumF32: return launch_wave<1, kLocalF32, kOutStream>(p, max_grid, s);
     case kOpHomSumI32: return launch_wave<1, kLocalI32, kOutStream>(p, max_grid, s);
     case kOpHomAdd: return launch_wave<2, kLocalNone, kOutStream>(p, max_grid, s);
-    default: return hipErrorInvalidValue;
-    }
-}
-
-hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
-{
-    switch (op) {
-    case kOpCompress: return launch_tile<0, kLocalF32, kOutStream>(p, max_grid, s);
-    case kOpDecompress: return launch_tile<1, kLocalNone, kOutF32>(p, max_grid, s);
-    case kOpHomSumF32: return launch_tile<1, kLocalF32, kOutStream>(p, max_grid, s);
-    case kOpHomSumI32: return launch_tile<1, kLocalI32, kOutStream>(p, max_grid, s);
-    case kOpHomAdd: return launch_tile<2, kLocalNone, kOutStream>(p, max_grid, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -10,12 +10,9 @@ enum : int { kLocalNone = 0, kLocalF32 = 1, kLocalI32 = 2 };   // local operand 
 enum : int { kOutStream = 0, kOutF32 = 1 };                    // what a tile produces
 enum : int { kOpCompress = 0, kOpDecompress, kOpHomSumF32, kOpHomSumI32, kOpHomAdd, kOpCount };
 
-// Tile geometry, shared by host and device: a workgroup of 256 lanes handles 8 elements per lane
-// per iteration.
-#ifndef HC_ITER
-#define HC_ITER 2
-#endif
-constexpr uint32_t kHostTileElems = 256u * 8u * HC_ITER;
+// Tile geometry, shared by host and device: a tile is 128 blocks of 32 elements; a wave handles
+// it in 8 sub-steps of 16 blocks (8 elements per lane, 4 lanes per block).
+constexpr uint32_t kHostTileElems = 4096;
 constexpr uint32_t kHostTileBlocks = kHostTileElems / 32u;
 constexpr uint32_t kHostChunkElems = 32768;
 
@@ -38,15 +35,14 @@ struct TileParams {
     uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
     uint64_t *total;            // receives the stream length
     uint64_t *user_total;       // optional second destination for the stream length
-    uint8_t *spill;             // wave kernels: kSpillSlotBytes per data wave and buffer for tiles that outgrow LDS
+    uint8_t *spill;             // kSpillSlotBytes per data wave and buffer, for tiles that outgrow the LDS stage
 };
 
-// Resident workgroups per compute unit for one of the tile kernels (sizes the persistent grid).
-hipError_t tile_kernel_residency(int op, int *blocks_per_cu);
-hipError_t launch_tile_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
-hipError_t wave_kernel_residency(int op, int *blocks_per_cu);
-hipError_t launch_wave_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
+// Bytes per data wave and buffer in the spill area (TileParams::spill): a whole worst-case tile.
 constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
+// Resident workgroups per compute unit of the kernel behind an operation (sizes the persistent grid).
+hipError_t op_kernel_residency(int op, int *blocks_per_cu);
+hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
 // Tile payload offsets of an incoming stream from its header bytes.
 hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
                              uint32_t *block_sums, uint64_t *ofs, hipStream_t s);
