@@ -108,6 +108,8 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, hipStream_t s)
 {
     p.spill = ws->d_spill;
+    p.out_slots = 2;
+    if (const char *e = std::getenv("HOMCOMP_SLOTS")) p.out_slots = std::strtol(e, nullptr, 10) == 4 ? 4u : 2u;
     return hip_ok(hc::launch_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -208,10 +210,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (op != hc::kOpDecompress && ws->max_grid[op] > widest) widest = ws->max_grid[op];
     }
     if (ok) {
-        // two spill slots per data wave of the widest encoder grid, no more waves than tiles
+        // four spill slots per data wave of the widest encoder grid, no more waves than tiles
         size_t waves = (size_t)(widest > 1 ? widest - 1 : 1) * 4;
         if (waves > ws->max_tiles) waves = ws->max_tiles;
-        ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 2 * hc::kSpillSlotBytes));
+        ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 4 * hc::kSpillSlotBytes));
     }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {

@@ -13,6 +13,9 @@
 
 #include "homcomp_kernels.hpp"
 
+#ifndef HC_POLL_SLEEP
+#define HC_POLL_SLEEP 64
+#endif
 namespace hc {
 
 constexpr int kWG = 256;                              // threads per workgroup (4 independent waves)
@@ -349,13 +352,14 @@ struct ScanCtx {
     uint32_t *err;
 };
 
+template <int SLEEP = 1>
 __device__ __forceinline__ bool scan_give_up(const ScanCtx &c, uint32_t &spins)
 {
     if (++spins > c.spin_limit) {
         atomicOr(c.err, 1u);
         return true;
     }
-    __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_s_sleep(SLEEP);
     return false;
 }
 
@@ -375,8 +379,11 @@ __device__ __forceinline__ uint64_t scan_probe(const ScanCtx &c, uint32_t tile)
 __device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint64_t w)
 {
     uint32_t spins = 0;
+    // Thousands of waves may wait here at the same time, for words that share a few cache lines
+    // with the words the scan server is writing: the pause between two looks keeps them from
+    // crowding the server out of those lines (HC_POLL_SLEEP x 64 clocks).
     while (status_state(w, c.epoch) != 2u) {
-        if (scan_give_up(c, spins)) break;
+        if (scan_give_up<HC_POLL_SLEEP>(c, spins)) break;
         w = scan_probe(c, tile);
     }
     return w & kValueMask;

@@ -6,6 +6,8 @@
 // blocks and belongs to one wave; the scan-server workgroup of the same launch turns the tiles'
 // byte totals into their offsets in the outgoing stream.  Small streaming kernels cover the
 // incoming-stream offsets, the Lorenzo pre-pass and the value range.
+#include <type_traits>
+
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
@@ -59,51 +61,84 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
 // the tile 2G after it (the step could not complete before the workgroup that waits for it has
 // published), i.e. a step covers at most 2G tiles: 1024 tiles (4 per lane) when G >= 512,
 // otherwise one tile per lane on min(256, 2G) lanes.
-__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
+// Pace of the server: the status words travel between compute units through memory, and while
+// the data waves keep the memory system busy such a trip takes several microseconds; every tile
+// passes through here, so the server must not pay one trip per step.  The totals of a step are
+// requested two steps ahead into two register sets used alternately, the request goes out ahead
+// of the step's own prefix stores, and the wave waits for exactly the loads it needs: a wave's
+// memory operations complete in issue order, so "all but the N youngest" leaves the later request
+// and the stores in flight.  The compiler cannot count memory operations across the retry loop
+// (it waits for everything), so the server issues its memory operations and waits by hand; every
+// one of them is issued unconditionally (lanes beyond the end load the last tiles' words again
+// and store into spare words), which makes the counts fixed.  With four tiles per lane the words
+// move in 16-byte pieces, two status words each (an aligned 8-byte word is never torn): two
+// loads and two stores per lane and step.
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+
+template <int PER>
+__device__ __forceinline__ void server_request(const uint64_t *src, uint64_t (&w)[PER])
 {
+    if constexpr (PER == 4) {
+        u64x2 a, b;
+        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(a) : "v"(src) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:16 sc1" : "=&v"(b) : "v"(src) : "memory");
+        w[0] = a.x; w[1] = a.y; w[2] = b.x; w[3] = b.y;
+    } else {
+        asm volatile("global_load_dwordx2 %0, %1, off sc1" : "=&v"(w[0]) : "v"(src) : "memory");
+    }
+}
+
+// Waits until at most N of the wave's memory operations are outstanding; the loaded words pass
+// through so that nothing reads them earlier.
+template <int N, int PER>
+__device__ __forceinline__ void server_wait(uint64_t (&w)[PER])
+{
+    static_assert(PER == 1 || PER == 4, "one asm statement per supported size");
+    if constexpr (PER == 4)
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]) : "n"(N) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(w[0]) : "n"(N) : "memory");
+}
+
+template <int PER>
+__device__ __forceinline__ void scan_server_steps(const TileParams &p, const ScanCtx &c, uint32_t lanes)
+{
+    constexpr int kOps = PER == 4 ? 2 : 1;   // memory instructions per request, and per step's stores
     __shared__ uint32_t s_wave[kWG / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const uint32_t per = G >= 512u ? 4u : 1u;                                   // tiles per lane
-    const uint32_t lanes = G >= 512u ? (uint32_t)kWG : (2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
-    const uint32_t step = per * lanes;
+    const uint32_t n = c.n_tiles;
+    const uint32_t step = PER * lanes;
     uint64_t base = 0;
-    // The totals of a step are requested two steps ahead, into two register sets used
-    // alternately: in the steady state they were published a round ago, so the server runs at the
-    // pace of its arithmetic instead of one memory round trip per step.  Lanes beyond the end
-    // request the last tiles again (no branch around the loads) and ignore what they get.
-    const uint32_t last = c.n_tiles - per;
-    auto request = [&](uint32_t t0, uint64_t (&dst)[4]) __attribute__((always_inline)) {
-        uint32_t idx = t0 + (uint32_t)tid * per;
+    const uint32_t last = n - PER;   // the number of tiles is a multiple of 8
+    auto request = [&](uint32_t t0, uint64_t (&w)[PER]) __attribute__((always_inline)) {
+        uint32_t idx = t0 + (uint32_t)tid * PER;
         if (idx > last) idx = last;
-        dst[0] = status_load(&c.totals[idx]);
-        if (per == 4u) {
-            dst[1] = status_load(&c.totals[idx + 1]);
-            dst[2] = status_load(&c.totals[idx + 2]);
-            dst[3] = status_load(&c.totals[idx + 3]);
-        }
+        server_request<PER>(c.totals + idx, w);
     };
-    auto process = [&](uint32_t t0, uint64_t (&w)[4]) __attribute__((always_inline)) {
-        const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
-        const bool in = (uint32_t)tid < lanes && idx < c.n_tiles;
-        if (in) {
-            uint32_t spins = 0;
-            for (;;) {
-                bool ok = status_state(w[0], c.epoch) == 1u;
-                if (per == 4u)
-                    ok = ok && status_state(w[1], c.epoch) == 1u && status_state(w[2], c.epoch) == 1u &&
-                         status_state(w[3], c.epoch) == 1u;
-                if (ok || scan_give_up(c, spins)) break;
-                request(t0, w);
-            }
-        }
-        uint32_t v[4], mine = 0;
+    // kYoung: memory instructions of this wave issued after the request for this step
+    auto process = [&](uint32_t t0, uint64_t (&w)[PER], auto young) __attribute__((always_inline)) {
+        constexpr int kYoung = decltype(young)::value;
+        const uint32_t idx = t0 + (uint32_t)tid * PER;
+        const bool in = (uint32_t)tid < lanes && idx < n;
+        server_wait<kYoung, PER>(w);
+        uint32_t spins = 0;
+        for (;;) {
+            bool ok = true;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            v[j] = in && j < per ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+            for (int j = 0; j < PER; ++j) ok = ok && (!in || status_state(w[j], c.epoch) == 1u);
+            if (ok || scan_give_up(c, spins)) break;
+            request(t0, w);
+            server_wait<0, PER>(w);
+        }
+        uint32_t v[PER], mine = 0;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
             mine += v[j];
         }
+        request(t0 + 2u * step, w);   // the set is free again; ahead of the stores below
         const uint32_t incl = wave_incl_scan_u32(mine, lane);
         if (lane == 63) s_wave[wave] = incl;
         __syncthreads();
@@ -114,34 +149,50 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
             if (q < wave) before += t;
             step_total += t;
         }
-        if (in) {
-            uint64_t run = base + before + (incl - mine);
+        uint64_t run = base + before + (incl - mine);
+        uint64_t out[PER];
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                if (j < per) {
-                    status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
-                    run += v[j];
-                }
-            }
+        for (int j = 0; j < PER; ++j) {
+            out[j] = status_word(c.epoch, 2, run);
+            run += v[j];
+        }
+        // lanes outside the step store into spare words next to the length word instead, so that
+        // the number of stores is fixed
+        uint64_t *const dst = in ? c.prefixes + idx : p.total + 4;
+        if constexpr (PER == 4) {
+            const u64x2 a = {out[0], out[1]}, b = {out[2], out[3]};
+            asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(a) : "memory");
+            asm volatile("global_store_dwordx4 %0, %1, off offset:16 sc1" : : "v"(dst), "v"(b) : "memory");
+        } else {
+            asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(dst), "v"(out[0]) : "memory");
         }
         base += step_total;
         __syncthreads();   // s_wave is reused by the next step
     };
-    uint64_t wa[4] = {0, 0, 0, 0}, wb[4] = {0, 0, 0, 0};
+    uint64_t wa[PER], wb[PER];
     request(0, wa);
     request(step, wb);
-    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += 2 * step) {
-        process(t0, wa);
-        request(t0 + 2 * step, wa);
-        if (t0 + step >= c.n_tiles) break;
-        process(t0 + step, wb);
-        request(t0 + 3 * step, wb);
+    // younger than the first step's request: the second request; from then on: the other set's
+    // request and one step's stores
+    process(0, wa, std::integral_constant<int, kOps>{});
+    for (uint32_t t0 = step; t0 < n; t0 += 2 * step) {
+        process(t0, wb, std::integral_constant<int, 2 * kOps>{});
+        if (t0 + step >= n) break;
+        process(t0 + step, wa, std::integral_constant<int, 2 * kOps>{});
     }
     if (tid == 0) {
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
         *p.total = len;
         if (p.user_total) *p.user_total = len;
     }
+}
+
+__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
+{
+    if (G >= 512u)
+        scan_server_steps<4>(p, c, kWG);
+    else
+        scan_server_steps<1>(p, c, 2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
 }
 
 // ---------------------------------------------------------------- wave-autonomous kernels
@@ -377,29 +428,47 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
 #pragma unroll
     for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j]);
 
-    uint32_t total1 = 0, total2 = 0;   // byte totals of the tiles of the previous two rounds
-    bool spilled1 = false, spilled2 = false;
-    uint64_t probe = 0;                // prefix word of the older one, requested a round ago
+    // Deferred tiles: a tile packed in round r is copied out in round r + D (D = p.out_slots, 2 to
+    // 4): its total is published when it is packed, the prefix word is requested in round
+    // r + D - 1 and used at the start of round r + D.  The wave's LDS stage is cut into D slots;
+    // more, smaller slots give the scan more time to come back (the words travel through memory,
+    // several microseconds each way under load) at the price of spilling tiles beyond a slot.
+    const int D = (int)p.out_slots;
+    const uint32_t slot_bytes = ((uint32_t)(2 * (kCap + 64)) / (uint32_t)D) & ~15u;
+    const uint32_t slot_cap = slot_bytes - 64u;
+    uint32_t tot[4] = {0, 0, 0, 0};     // byte totals of the tiles of the previous rounds, newest first
+    bool spl[4] = {false, false, false, false};
+    uint64_t probe = 0;                // prefix word of the oldest one, requested a round ago
 
     for (int64_t r = 0;; ++r) {
-        const int64_t t0 = tile_of(r), t1 = t0 - GW, t2 = t0 - 2 * GW;
+        const int64_t t0 = tile_of(r);
+        const int64_t tp = t0 - (int64_t)(D - 1) * GW;   // its prefix is requested at the end of this round
+        const int64_t td = t0 - (int64_t)D * GW;         // copied out at the start of this round
         const bool v0 = t0 < n_tiles;
-        const bool v1 = kEnc && r >= 1 && t1 < n_tiles;
-        const bool v2 = kEnc && r >= 2 && t2 < n_tiles;
-        if (!v0 && !v1 && !v2) break;
+        const bool vp = kEnc && r >= D - 1 && tp < n_tiles;
+        const bool vd = kEnc && r >= D && td < n_tiles;
+        if (!v0 && (!kEnc || td >= n_tiles)) break;
         const int buf = (int)(r & 1);
-        uint8_t *stage = s_out[wave][buf];
-        uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * 2u + (uint64_t)buf) * kSpillSlotBytes : nullptr;
+        const int obuf = (int)(r % D);
+        uint8_t *stage = &s_out[wave][0][0] + (uint32_t)obuf * slot_bytes;
+        uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * 4u + (uint64_t)obuf) * kSpillSlotBytes : nullptr;
 
-        // ---- the tile packed two rounds ago goes to its place in the stream
+        // ---- the tile packed D rounds ago goes to its place in the stream
         if constexpr (kEnc) {
-            if (v2) {
-                const uint64_t excl = scan_resolve(scan, (uint32_t)t2, probe);
+            if (vd) {
+                const uint32_t total_d = D == 2 ? tot[1] : (D == 3 ? tot[2] : tot[3]);
+                const bool spilled_d = D == 2 ? spl[1] : (D == 3 ? spl[2] : spl[3]);
+                // the prefix word travels in lane 0 only: a device-scope load is executed per
+                // lane, so 64 lanes asking for the same word would be 64 requests
+                uint64_t excl = 0;
+                if (lane == 0) excl = scan_resolve(scan, (uint32_t)td, probe);
+                excl = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(excl >> 32)) << 32) |
+                       (uint32_t)__builtin_amdgcn_readfirstlane((int)excl);
                 uint8_t *dst = p.out_cmp + p.hdr_bytes + excl;
-                if (spilled2)
-                    copy_out_spill(slot, dst, total2, lane);
+                if (spilled_d)
+                    copy_out_spill(slot, dst, total_d, lane);
                 else
-                    copy_out<64>(stage, dst, total2, lane);
+                    copy_out<64>(stage, dst, total_d, lane);
             }
         }
 
@@ -503,7 +572,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     const uint32_t pos = run + incl - size;
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
-                    if (!spilled0 && run + sub_total > (uint32_t)kCap) {
+                    if (!spilled0 && run + sub_total > slot_cap) {
                         // the tile outgrows the LDS stage: what is packed so far moves to the spill slot
                         for (uint32_t i = 4u * lane; i < run; i += 256u)
                             *reinterpret_cast<uint32_t *>(slot + i) = *reinterpret_cast<const uint32_t *>(stage + i);
@@ -536,11 +605,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             }
         }
         if constexpr (kEnc) {
-            if (v1) probe = scan_probe(scan, (uint32_t)t1);
-            total2 = total1;
-            total1 = run;
-            spilled2 = spilled1;
-            spilled1 = spilled0;
+            if (vp && lane == 0) probe = scan_probe(scan, (uint32_t)tp);
+            tot[3] = tot[2]; tot[2] = tot[1]; tot[1] = tot[0]; tot[0] = run;
+            spl[3] = spl[2]; spl[2] = spl[1]; spl[1] = spl[0]; spl[0] = spilled0;
         }
     }
 }

@@ -35,10 +35,11 @@ struct TileParams {
     uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
     uint64_t *total;            // receives the stream length
     uint64_t *user_total;       // optional second destination for the stream length
-    uint8_t *spill;             // kSpillSlotBytes per data wave and buffer, for tiles that outgrow the LDS stage
+    uint8_t *spill;             // four slots of kSpillSlotBytes per data wave, for tiles that outgrow their LDS slot
+    uint32_t out_slots;         // rounds a packed tile waits in LDS for its stream offset: 2 or 4
 };
 
-// Bytes per data wave and buffer in the spill area (TileParams::spill): a whole worst-case tile.
+// Bytes per slot of the spill area (TileParams::spill): a whole worst-case tile.
 constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
 // Resident workgroups per compute unit of the kernel behind an operation (sizes the persistent grid).
 hipError_t op_kernel_residency(int op, int *blocks_per_cu);
