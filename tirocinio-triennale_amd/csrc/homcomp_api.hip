@@ -53,7 +53,8 @@ struct homcomp_workspace {
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
     uint32_t max_grid[hc::kOpCount];  // workgroups of each operation's kernel that this device keeps resident
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
-    uint8_t *d_spill;         // spill slots: two worst-case tiles per data wave
+    uint8_t *d_spill;         // spill slots: four worst-case tiles per data wave
+    uint32_t out_slots;       // deferral depth of packed tiles (2..4)
 };
 
 namespace {
@@ -108,8 +109,10 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, hipStream_t s)
 {
     p.spill = ws->d_spill;
-    p.out_slots = 2;
-    if (const char *e = std::getenv("HOMCOMP_SLOTS")) p.out_slots = std::strtol(e, nullptr, 10) == 4 ? 4u : 2u;
+    // Rounds a packed tile waits in LDS for its stream offset.  More rounds give the offset scan
+    // more time, but cut the LDS stage of a wave into smaller slots, and tiles beyond a slot take
+    // the slower path through the spill area.  HOMCOMP_SLOTS (2..4) overrides the default.
+    p.out_slots = ws->out_slots;
     return hip_ok(hc::launch_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -214,6 +217,11 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         size_t waves = (size_t)(widest > 1 ? widest - 1 : 1) * 4;
         if (waves > ws->max_tiles) waves = ws->max_tiles;
         ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 4 * hc::kSpillSlotBytes));
+    }
+    ws->out_slots = 2;
+    if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
+        const long v = std::strtol(e, nullptr, 10);
+        if (v >= 2 && v <= 4) ws->out_slots = (uint32_t)v;
     }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {

@@ -6,8 +6,6 @@
 // blocks and belongs to one wave; the scan-server workgroup of the same launch turns the tiles'
 // byte totals into their offsets in the outgoing stream.  Small streaming kernels cover the
 // incoming-stream offsets, the Lorenzo pre-pass and the value range.
-#include <type_traits>
-
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
@@ -61,84 +59,51 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
 // the tile 2G after it (the step could not complete before the workgroup that waits for it has
 // published), i.e. a step covers at most 2G tiles: 1024 tiles (4 per lane) when G >= 512,
 // otherwise one tile per lane on min(256, 2G) lanes.
-// Pace of the server: the status words travel between compute units through memory, and while
-// the data waves keep the memory system busy such a trip takes several microseconds; every tile
-// passes through here, so the server must not pay one trip per step.  The totals of a step are
-// requested two steps ahead into two register sets used alternately, the request goes out ahead
-// of the step's own prefix stores, and the wave waits for exactly the loads it needs: a wave's
-// memory operations complete in issue order, so "all but the N youngest" leaves the later request
-// and the stores in flight.  The compiler cannot count memory operations across the retry loop
-// (it waits for everything), so the server issues its memory operations and waits by hand; every
-// one of them is issued unconditionally (lanes beyond the end load the last tiles' words again
-// and store into spare words), which makes the counts fixed.  With four tiles per lane the words
-// move in 16-byte pieces, two status words each (an aligned 8-byte word is never torn): two
-// loads and two stores per lane and step.
-typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
-
-template <int PER>
-__device__ __forceinline__ void server_request(const uint64_t *src, uint64_t (&w)[PER])
+__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
 {
-    if constexpr (PER == 4) {
-        u64x2 a, b;
-        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(a) : "v"(src) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, off offset:16 sc1" : "=&v"(b) : "v"(src) : "memory");
-        w[0] = a.x; w[1] = a.y; w[2] = b.x; w[3] = b.y;
-    } else {
-        asm volatile("global_load_dwordx2 %0, %1, off sc1" : "=&v"(w[0]) : "v"(src) : "memory");
-    }
-}
-
-// Waits until at most N of the wave's memory operations are outstanding; the loaded words pass
-// through so that nothing reads them earlier.
-template <int N, int PER>
-__device__ __forceinline__ void server_wait(uint64_t (&w)[PER])
-{
-    static_assert(PER == 1 || PER == 4, "one asm statement per supported size");
-    if constexpr (PER == 4)
-        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]) : "n"(N) : "memory");
-    else
-        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(w[0]) : "n"(N) : "memory");
-}
-
-template <int PER>
-__device__ __forceinline__ void scan_server_steps(const TileParams &p, const ScanCtx &c, uint32_t lanes)
-{
-    constexpr int kOps = PER == 4 ? 2 : 1;   // memory instructions per request, and per step's stores
     __shared__ uint32_t s_wave[kWG / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const uint32_t n = c.n_tiles;
-    const uint32_t step = PER * lanes;
+    const uint32_t per = G >= 512u ? 4u : 1u;                                   // tiles per lane
+    const uint32_t lanes = G >= 512u ? (uint32_t)kWG : (2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
+    const uint32_t step = per * lanes;
     uint64_t base = 0;
-    const uint32_t last = n - PER;   // the number of tiles is a multiple of 8
-    auto request = [&](uint32_t t0, uint64_t (&w)[PER]) __attribute__((always_inline)) {
-        uint32_t idx = t0 + (uint32_t)tid * PER;
+    // The totals of a step are requested two steps ahead, into two register sets used
+    // alternately: in the steady state they were published a round ago, so the server runs at the
+    // pace of its arithmetic instead of one memory round trip per step.  Lanes beyond the end
+    // request the last tiles again (no branch around the loads) and ignore what they get.
+    const uint32_t last = c.n_tiles - per;
+    auto request = [&](uint32_t t0, uint64_t (&dst)[4]) __attribute__((always_inline)) {
+        uint32_t idx = t0 + (uint32_t)tid * per;
         if (idx > last) idx = last;
-        server_request<PER>(c.totals + idx, w);
-    };
-    // kYoung: memory instructions of this wave issued after the request for this step
-    auto process = [&](uint32_t t0, uint64_t (&w)[PER], auto young) __attribute__((always_inline)) {
-        constexpr int kYoung = decltype(young)::value;
-        const uint32_t idx = t0 + (uint32_t)tid * PER;
-        const bool in = (uint32_t)tid < lanes && idx < n;
-        server_wait<kYoung, PER>(w);
-        uint32_t spins = 0;
-        for (;;) {
-            bool ok = true;
-#pragma unroll
-            for (int j = 0; j < PER; ++j) ok = ok && (!in || status_state(w[j], c.epoch) == 1u);
-            if (ok || scan_give_up(c, spins)) break;
-            request(t0, w);
-            server_wait<0, PER>(w);
+        dst[0] = status_load(&c.totals[idx]);
+        if (per == 4u) {
+            dst[1] = status_load(&c.totals[idx + 1]);
+            dst[2] = status_load(&c.totals[idx + 2]);
+            dst[3] = status_load(&c.totals[idx + 3]);
         }
-        uint32_t v[PER], mine = 0;
+    };
+    auto process = [&](uint32_t t0, uint64_t (&w)[4]) __attribute__((always_inline)) {
+        const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
+        const bool in = (uint32_t)tid < lanes && idx < c.n_tiles;
+        if (in) {
+            uint32_t spins = 0;
+            for (;;) {
+                bool ok = status_state(w[0], c.epoch) == 1u;
+                if (per == 4u)
+                    ok = ok && status_state(w[1], c.epoch) == 1u && status_state(w[2], c.epoch) == 1u &&
+                         status_state(w[3], c.epoch) == 1u;
+                if (ok || scan_give_up(c, spins)) break;
+                request(t0, w);
+            }
+        }
+        uint32_t v[4], mine = 0;
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+        for (uint32_t j = 0; j < 4; ++j) {
+            v[j] = in && j < per ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
             mine += v[j];
         }
-        request(t0 + 2u * step, w);   // the set is free again; ahead of the stores below
         const uint32_t incl = wave_incl_scan_u32(mine, lane);
         if (lane == 63) s_wave[wave] = incl;
         __syncthreads();
@@ -149,50 +114,34 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
             if (q < wave) before += t;
             step_total += t;
         }
-        uint64_t run = base + before + (incl - mine);
-        uint64_t out[PER];
+        if (in) {
+            uint64_t run = base + before + (incl - mine);
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            out[j] = status_word(c.epoch, 2, run);
-            run += v[j];
-        }
-        // lanes outside the step store into spare words next to the length word instead, so that
-        // the number of stores is fixed
-        uint64_t *const dst = in ? c.prefixes + idx : p.total + 4;
-        if constexpr (PER == 4) {
-            const u64x2 a = {out[0], out[1]}, b = {out[2], out[3]};
-            asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(a) : "memory");
-            asm volatile("global_store_dwordx4 %0, %1, off offset:16 sc1" : : "v"(dst), "v"(b) : "memory");
-        } else {
-            asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(dst), "v"(out[0]) : "memory");
+            for (uint32_t j = 0; j < 4; ++j) {
+                if (j < per) {
+                    status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
+                    run += v[j];
+                }
+            }
         }
         base += step_total;
         __syncthreads();   // s_wave is reused by the next step
     };
-    uint64_t wa[PER], wb[PER];
+    uint64_t wa[4] = {0, 0, 0, 0}, wb[4] = {0, 0, 0, 0};
     request(0, wa);
     request(step, wb);
-    // younger than the first step's request: the second request; from then on: the other set's
-    // request and one step's stores
-    process(0, wa, std::integral_constant<int, kOps>{});
-    for (uint32_t t0 = step; t0 < n; t0 += 2 * step) {
-        process(t0, wb, std::integral_constant<int, 2 * kOps>{});
-        if (t0 + step >= n) break;
-        process(t0 + step, wa, std::integral_constant<int, 2 * kOps>{});
+    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += 2 * step) {
+        process(t0, wa);
+        request(t0 + 2 * step, wa);
+        if (t0 + step >= c.n_tiles) break;
+        process(t0 + step, wb);
+        request(t0 + 3 * step, wb);
     }
     if (tid == 0) {
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
         *p.total = len;
         if (p.user_total) *p.user_total = len;
     }
-}
-
-__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
-{
-    if (G >= 512u)
-        scan_server_steps<4>(p, c, kWG);
-    else
-        scan_server_steps<1>(p, c, 2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
 }
 
 // ---------------------------------------------------------------- wave-autonomous kernels
