@@ -72,6 +72,46 @@ def cpu_baseline(orc, x_np, y_np, eb, budget_s: float = 20.0):
     }, sa, ss
 
 
+def sweep(torch, pkg, gen) -> int:
+    """Sizes 2^20..2^28 x {smooth, gradient-like, uniform} x REL {1e-2, 1e-4, 1e-6}: kernel-side
+    time of compress, decompress, hom_sum_f32 and hom_add, compression ratio, fraction of HBM peak."""
+    for log2n in (20, 22, 24, 26, 28):
+        n = 1 << log2n
+        ws = pkg.Workspace(n)
+        cap = pkg.max_stream_bytes(n)
+        bufs = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(3)]
+        dec = torch.empty(n, dtype=torch.float32, device="cuda")
+        mm = torch.empty(4, dtype=torch.float32, device="cuda")
+        for kind in ("smooth", "gradient_like", "uniform"):
+            x = gen.GENERATORS_TORCH[kind](n, seed=1)
+            y = gen.GENERATORS_TORCH[kind](n, seed=2)
+            ws.value_range(x, mm[0:2])
+            ws.value_range(y, mm[2:4])
+            r = mm.cpu().numpy()
+            for rel in (1e-2, 1e-4, 1e-6):
+                eb = pkg.rel_to_abs(rel, float(min(r[0], r[2])), float(max(r[1], r[3])))
+                ca, cb, cs = bufs
+                ws.compress(x, eb, ca)
+                la = ws.last_size()
+                ws.compress(y, eb, cb)
+                lb = ws.last_size()
+                ws.hom_sum_f32(ca, la, y, eb, cs)
+                ls = ws.last_size()
+                it = 20 if log2n <= 24 else 8
+                t_c = time_op(torch, lambda: ws.compress(x, eb, ca), it)
+                t_h = time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), it)
+                t_d = time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), it)
+                t_a = time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, cs), it)
+                pt = {"log2n": log2n, "kind": kind, "rel": rel, "CR": round(4 * n / la, 2), "CR_sum": round(4 * n / ls, 2)}
+                for name, ms, alg in (("compress", t_c, 4 * n + la), ("hom_sum_f32", t_h, la + 4 * n + ls),
+                                      ("decompress", t_d, ls + 4 * n), ("hom_add", t_a, la + lb + ls)):
+                    pt[name] = {"us": round(ms * 1e3, 1), "GBps_input": round(4 * n / ms / 1e6, 1),
+                                "frac_hbm": round(alg / (ms * 1e-3) / HBM_PEAK, 4)}
+                print(json.dumps(pt), flush=True)
+        del ws
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -85,6 +125,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1:1 copy of an operand (reference point for HBM counters)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark line: sizes x data families x REL bounds, one JSON line per point")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; --gpus above 1 is not part of this build "
@@ -97,6 +139,8 @@ def main() -> int:
     pkg = entry.load_package()
     gen = entry.load_datagen()
     torch.cuda.set_device(0)
+    if args.sweep:
+        return sweep(torch, pkg, gen)
     n = 1 << args.log2n
     x = gen.GENERATORS_TORCH[args.kind](n, seed=1)
     y = gen.GENERATORS_TORCH[args.kind](n, seed=2)

@@ -291,3 +291,46 @@ def test_many_rounds_and_small_grids(pkg, cuda, orc, gen, monkeypatch, grid_perc
         assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
     finally:
         g.close()
+
+
+@pytest.mark.parametrize("stage,slots", [("small", 2), ("large", 2), ("small", 3), ("small", 4), ("large", 4)])
+def test_lds_budgets_and_deferral_depths(pkg, cuda, orc, gen, monkeypatch, stage, slots):
+    """Every LDS budget (HOMCOMP_STAGE) and deferral depth (HOMCOMP_SLOTS) gives the same bytes:
+    with the small budget and many slots most tiles of poorly compressible data outgrow their LDS
+    slot and travel through the spill area, with the large one they stay in LDS."""
+    monkeypatch.setenv("HOMCOMP_STAGE", stage)
+    monkeypatch.setenv("HOMCOMP_SLOTS", str(slots))
+    orc.set_threads(16)
+    n = (1 << 22) + 4099   # many rounds per wave, ragged end
+    for a, b, eb in ((gen.uniform_np(n, 41), gen.uniform_np(n, 42), np.float32(1e-5)),        # ~60 B per block: spills everywhere
+                     (gen.smooth_np(n, 43), gen.smooth_np(n, 44), np.float32(8e-4)),         # ~15 B per block: stays in LDS
+                     (gen.gradient_like_np(n, 45), gen.uniform_np(n, 46), np.float32(1e-4))):  # mixed tile sizes
+        g = Gpu(pkg, cuda, n)
+        try:
+            sa = g.compress(a, eb)
+            assert_stream_equal(sa, orc.compress(a, eb), "compress")
+            sb = g.compress(b, eb)
+            want = orc.hom_sum_f32(sa, b, eb)
+            assert_stream_equal(g.hom_sum_f32(sa, b, eb), want, "hom_sum_f32")
+            assert_stream_equal(g.hom_add(sa, sb, n), want, "hom_add")
+            # int32 deltas end with the array (the float path pads with 0.0f, whose delta is -q[n-1])
+            qp = orc.quant_predict(b, eb)
+            assert_stream_equal(g.hom_sum_i32(sa, qp), orc.hom_sum_i32(sa, qp), "hom_sum_i32")
+        finally:
+            g.close()
+
+
+def test_lds_budget_follows_the_data(pkg, cuda, orc, gen):
+    """Without a forced budget a workspace starts compress with the large LDS budget and moves to
+    the small one once a finished call has shown the data to be compressible; alternating data
+    families on one workspace must keep producing the oracle's bytes."""
+    orc.set_threads(16)
+    n = 1 << 21
+    g = Gpu(pkg, cuda, n)
+    try:
+        for seed, (maker, eb) in enumerate([(gen.smooth_np, 8e-4), (gen.smooth_np, 8e-4), (gen.uniform_np, 1e-5),
+                                            (gen.uniform_np, 1e-5), (gen.smooth_np, 8e-4), (gen.gradient_like_np, 1e-6)]):
+            x = maker(n, 50 + seed)
+            assert_stream_equal(g.compress(x, np.float32(eb)), orc.compress(x, np.float32(eb)), f"compress #{seed}")
+    finally:
+        g.close()

@@ -51,10 +51,12 @@ struct homcomp_workspace {
     float *d_partial;         // min/max partials
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
-    uint32_t max_grid[hc::kOpCount];  // workgroups of each operation's kernel that this device keeps resident
+    uint32_t max_grid[hc::kOpCount][2];  // resident workgroups of each operation's kernel, per LDS budget (small, large)
+    uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint8_t *d_spill;         // spill slots: four worst-case tiles per data wave
     uint32_t out_slots;       // deferral depth of packed tiles (2..4)
+    int stage_class;          // -1: chosen per call; 0 / 1: HOMCOMP_STAGE=small / large forces one LDS budget
 };
 
 namespace {
@@ -106,14 +108,36 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
                : HOMCOMP_ERR_HIP;
 }
 
-int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, hipStream_t s)
+// LDS stage per data wave (two deferred tiles by default).  The small budgets fit tiles of streams
+// compressed about 4x or better and let more waves share a compute unit; the large one holds
+// tiles down to a ratio of 2.  A tile beyond its slot still works (it goes through the spill
+// area), only slower, so the choice below is a performance heuristic, never a correctness matter.
+constexpr uint32_t kStageSmall[hc::kOpCount] = {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)};
+constexpr uint32_t kStageLarge = 2 * (8192 + 64);
+
+// expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
+int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
     p.spill = ws->d_spill;
-    // Rounds a packed tile waits in LDS for its stream offset.  More rounds give the offset scan
-    // more time, but cut the LDS stage of a wave into smaller slots, and tiles beyond a slot take
-    // the slower path through the spill area.  HOMCOMP_SLOTS (2..4) overrides the default.
     p.out_slots = ws->out_slots;
-    return hip_ok(hc::launch_op(op, p, ws->max_grid[op], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    int cls = 1;
+    if (op == hc::kOpDecompress) {
+        cls = 0;
+    } else {
+        if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
+        const uint64_t slot_cap = kStageSmall[op] / ws->out_slots - 64u;
+        if (expected_tile_bytes != 0 && expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) cls = 0;
+        if (ws->stage_class >= 0) cls = ws->stage_class;
+        p.host_total = &ws->h_mean_tile[op];
+    }
+    p.stage_bytes = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge : kStageSmall[op]);
+    return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+}
+
+// payload bytes per tile of an incoming stream
+uint64_t tile_bytes_of(const hc::TileParams &p, size_t stream_size)
+{
+    return stream_size > p.hdr_bytes ? (stream_size - p.hdr_bytes) / p.n_tiles : 1u;
 }
 
 // n == 0: the stream is empty; only the length words are written.
@@ -196,27 +220,36 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     bool ok = hip_ok(hipGetDeviceProperties(&prop, ws->device));
     uint32_t widest = 0;
     for (int op = 0; ok && op < hc::kOpCount; ++op) {
-        int per_cu = 0;
-        ok = hip_ok(hc::op_kernel_residency(op, &per_cu));
-        if (ok && per_cu < 1) per_cu = 1;
-        // one compute unit's worth of workgroups is left free: the persistent grid must be fully
-        // resident, and an estimate that is off by a single workgroup would stall the launch
-        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
-        ws->max_grid[op] = (uint32_t)per_cu * (uint32_t)cus;
-        // HOMCOMP_GRID_PERCENT (1..100) shrinks the persistent grid, for devices that are shared
-        // with other work and cannot keep a full grid of this library resident
-        if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
-            const long pct = std::strtol(e, nullptr, 10);
-            if (pct >= 1 && pct <= 100) ws->max_grid[op] = (uint32_t)((uint64_t)ws->max_grid[op] * (uint64_t)pct / 100u);
+        for (int cls = 0; ok && cls < 2; ++cls) {
+            int per_cu = 0;
+            const uint32_t stage = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge : kStageSmall[op]);
+            ok = hip_ok(hc::op_kernel_residency(op, stage, &per_cu));
+            if (ok && per_cu < 1) per_cu = 1;
+            // one compute unit's worth of workgroups is left free: the persistent grid must be fully
+            // resident, and an estimate that is off by a single workgroup would stall the launch
+            const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
+            uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
+            // HOMCOMP_GRID_PERCENT (1..100) shrinks the persistent grid, for devices that are shared
+            // with other work and cannot keep a full grid of this library resident
+            if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
+                const long pct = std::strtol(e, nullptr, 10);
+                if (pct >= 1 && pct <= 100) g = (uint32_t)((uint64_t)g * (uint64_t)pct / 100u);
+            }
+            if (g < 2) g = 2;   // an encoder needs a data workgroup and the scan server
+            ws->max_grid[op][cls] = g;
+            if (op != hc::kOpDecompress && g > widest) widest = g;
         }
-        if (ws->max_grid[op] < 2) ws->max_grid[op] = 2;   // an encoder needs a data workgroup and the scan server
-        if (op != hc::kOpDecompress && ws->max_grid[op] > widest) widest = ws->max_grid[op];
     }
     if (ok) {
         // four spill slots per data wave of the widest encoder grid, no more waves than tiles
         size_t waves = (size_t)(widest > 1 ? widest - 1 : 1) * 4;
         if (waves > ws->max_tiles) waves = ws->max_tiles;
         ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 4 * hc::kSpillSlotBytes));
+    }
+    ws->stage_class = -1;
+    if (const char *e = std::getenv("HOMCOMP_STAGE")) {
+        if (std::strcmp(e, "small") == 0) ws->stage_class = 0;
+        if (std::strcmp(e, "large") == 0) ws->stage_class = 1;
     }
     ws->out_slots = 2;
     if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
@@ -229,12 +262,14 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (v >= 1 && v <= (1l << 30)) ws->spin_limit = (uint32_t)v;
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
-        !hip_ok(hipHostMalloc((void **)&ws->h_total, 2 * sizeof(uint64_t), hipHostMallocDefault))) {
+        !hip_ok(hipHostMalloc((void **)&ws->h_total, (2 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
         if (ws->d_spill) (void)hipFree(ws->d_spill);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
+    std::memset(ws->h_total, 0, (2 + hc::kOpCount) * sizeof(uint64_t));
+    ws->h_mean_tile = ws->h_total + 2;
     uint8_t *base = (uint8_t *)ws->d_block;
     ws->d_tile_totals = (uint64_t *)(base + o_status);
     ws->d_tile_prefixes = ws->d_tile_totals + t;
@@ -278,7 +313,7 @@ int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEl
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    return run_tile_op(ws, hc::kOpCompress, p, s);
+    return run_tile_op(ws, hc::kOpCompress, p, 0, s);
 }
 
 int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
@@ -299,7 +334,7 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     if ((rc = in_offsets(ws, 0, d_cmp, &p, s))) return rc;
-    return run_tile_op(ws, hc::kOpDecompress, p, s);
+    return run_tile_op(ws, hc::kOpDecompress, p, 0, s);
 }
 
 int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
@@ -323,7 +358,7 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
     if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
-    return run_tile_op(ws, hc::kOpHomSumF32, p, s);
+    return run_tile_op(ws, hc::kOpHomSumF32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
 int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
@@ -344,7 +379,7 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
     if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
-    return run_tile_op(ws, hc::kOpHomSumI32, p, s);
+    return run_tile_op(ws, hc::kOpHomSumI32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
 int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t size_a,
@@ -366,7 +401,8 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
     p.user_total = d_stream_len;
     if ((rc = in_offsets(ws, 0, d_cmp_a, &p, s))) return rc;
     if ((rc = in_offsets(ws, 1, d_cmp_b, &p, s))) return rc;
-    return run_tile_op(ws, hc::kOpHomAdd, p, s);
+    const uint64_t ta = tile_bytes_of(p, size_a), tb = tile_bytes_of(p, size_b);
+    return run_tile_op(ws, hc::kOpHomAdd, p, ta > tb ? ta : tb, s);
 }
 
 int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,

@@ -9,12 +9,6 @@
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
-#ifndef HC_CAP0
-#define HC_CAP0 4096
-#endif
-#ifndef HC_CAP1
-#define HC_CAP1 3072
-#endif
 #ifndef HC_DEPTH_ENC
 #define HC_DEPTH_ENC 2
 #endif
@@ -141,6 +135,8 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
         *p.total = len;
         if (p.user_total) *p.user_total = len;
+        // mean payload bytes per tile, for the host's choice of the next launch's LDS budget
+        if (p.host_total) *p.host_total = base / c.n_tiles;
     }
 }
 
@@ -163,14 +159,12 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
 // Stream output: rate selection, an in-wave DPP scan of the 16 block sizes, pack at the running
 // offset into the wave's LDS stage.  The tile's place in the stream comes from the scan server
 // (HomComp/src/GSZ.cu:170-239): total published when the tile is packed, prefix requested a
-// round later, payload copied out two rounds later.  The LDS stage of a deferred tile holds
-// wave_cap() bytes (the budget that lets 12-16 waves share a compute unit); a tile that outgrows
-// it continues in the wave's slot of a global spill area and is copied out from there.
+// round later, payload copied out two rounds later.  The LDS stage of a wave is sized by the launch
+// (a budget chosen from the expected compressed size: smaller stages let more waves share a
+// compute unit); a tile that outgrows its slot continues in the wave's slot of a global spill
+// area and is copied out from there.
 constexpr int kSub = kTileBlocks / 16;
 constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
-
-template <int NIN>
-constexpr int wave_cap() { return NIN == 0 ? HC_CAP0 : (NIN == 1 ? HC_CAP1 : 2048); }
 
 template <int LOCAL>
 struct SubRegs {
@@ -254,13 +248,14 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     constexpr bool kEnc = OUT == kOutStream;
     constexpr int kW = kWG / 64;
     constexpr int kIn = NIN > 0 ? NIN : 1;
-    constexpr int kCap = wave_cap<NIN>();
     // Sub-steps between a request and its use.  A wave's memory operations complete in order, so
     // waiting for a load also waits for every store issued before it: the decoder, which stores
     // 2 KiB per sub-step, looks further ahead to keep more of its stores in flight.
     constexpr int kDepth = HC_DEPTH_ENC > 0 && kEnc ? HC_DEPTH_ENC : 4;
     static_assert(kSub % kDepth == 0, "the register sets rotate with the sub-steps of a tile");
-    __shared__ __align__(16) uint8_t s_out[kW][2][kEnc ? kCap + 64 : 16];
+    // stage of the packed tiles that wait for their stream offset: p.stage_bytes per wave, sized by
+    // the launch (dynamic LDS), see TileParams
+    extern __shared__ __align__(16) uint8_t s_dyn[];
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
     __shared__ __align__(16) uint8_t s_in[kW][kIn][NIN > 0 ? kInStage : 16];
     __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
@@ -383,7 +378,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // more, smaller slots give the scan more time to come back (the words travel through memory,
     // several microseconds each way under load) at the price of spilling tiles beyond a slot.
     const int D = (int)p.out_slots;
-    const uint32_t slot_bytes = ((uint32_t)(2 * (kCap + 64)) / (uint32_t)D) & ~15u;
+    const uint32_t slot_bytes = (p.stage_bytes / (uint32_t)D) & ~15u;
     const uint32_t slot_cap = slot_bytes - 64u;
     uint32_t tot[4] = {0, 0, 0, 0};     // byte totals of the tiles of the previous rounds, newest first
     bool spl[4] = {false, false, false, false};
@@ -399,7 +394,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         if (!v0 && (!kEnc || td >= n_tiles)) break;
         const int buf = (int)(r & 1);
         const int obuf = (int)(r % D);
-        uint8_t *stage = &s_out[wave][0][0] + (uint32_t)obuf * slot_bytes;
+        uint8_t *stage = s_dyn + (uint32_t)wave * p.stage_bytes + (uint32_t)obuf * slot_bytes;
         uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * 4u + (uint64_t)obuf) * kSpillSlotBytes : nullptr;
 
         // ---- the tile packed D rounds ago goes to its place in the stream
@@ -778,24 +773,29 @@ static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_
     uint32_t grid = (p.n_tiles + 3u) / 4u + extra;
     if (grid > max_grid) grid = max_grid;
     if (grid < 1u + extra) grid = 1u + extra;
-    hipLaunchKernelGGL((k_wave<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), 0, s, p);
+    const uint32_t dyn = OUT == kOutStream ? (kWG / 64) * p.stage_bytes : 0u;
+    hipLaunchKernelGGL((k_wave<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), dyn, s, p);
     return hipGetLastError();
 }
 
 template <int NIN, int LOCAL, int OUT>
-static hipError_t wave_resident_blocks(int *blocks_per_cu)
+static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
 {
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, 0);
+    const size_t dyn = OUT == kOutStream ? (size_t)(kWG / 64) * stage_bytes : 0;
+    const void *fn = reinterpret_cast<const void *>(&k_wave<NIN, LOCAL, OUT>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+    if (e != hipSuccess) return e;
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, dyn);
 }
 
-hipError_t op_kernel_residency(int op, int *blocks_per_cu)
+hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu)
 {
     switch (op) {
-    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu);
-    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu);
-    case kOpHomSumF32: return wave_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu);
-    case kOpHomSumI32: return wave_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu);
-    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu);
+    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu, stage_bytes);
+    case kOpHomSumF32: return wave_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpHomSumI32: return wave_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu, stage_bytes);
     default: return hipErrorInvalidValue;
     }
 }

@@ -36,13 +36,15 @@ struct TileParams {
     uint64_t *total;            // receives the stream length
     uint64_t *user_total;       // optional second destination for the stream length
     uint8_t *spill;             // four slots of kSpillSlotBytes per data wave, for tiles that outgrow their LDS slot
-    uint32_t out_slots;         // rounds a packed tile waits in LDS for its stream offset: 2 or 4
+    uint32_t out_slots;         // rounds a packed tile waits in LDS for its stream offset: 2 to 4
+    uint32_t stage_bytes;       // LDS bytes per data wave for those tiles (a multiple of 64); cut into out_slots slots
+    uint64_t *host_total;       // optional pinned host word that also receives the stream length
 };
 
 // Bytes per slot of the spill area (TileParams::spill): a whole worst-case tile.
 constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
 // Resident workgroups per compute unit of the kernel behind an operation (sizes the persistent grid).
-hipError_t op_kernel_residency(int op, int *blocks_per_cu);
+hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu);
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
 // Tile payload offsets of an incoming stream from its header bytes.
 hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
