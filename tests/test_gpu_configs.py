@@ -117,3 +117,79 @@ def test_config4_ring_reduce_scatter(pkg, orc, gen, cuda):
         for h in host:
             exact += h[sl]
         assert (np.abs(dec - exact) <= ranks * float(eb) * (1 + 1e-3)).all()
+
+
+def ring_segments(count, ranks):
+    """Block offsets and counts of the segmented ring (HomComp/src/cuda_awareallreduce.cu:455-489):
+    blocks are cut from the count padded to 32768, rounded up to multiples of 4, and the last block
+    ends with the array."""
+    pad = (count + 32767) // 32768 * 32768
+    early = late = pad // ranks
+    split = pad % ranks
+    if split:
+        early += 1
+    early += (-early) % 4
+    late += (-late) % 4
+    offs, cnts = [], []
+    for b in range(ranks):
+        off = b * early if b < split else split * early + (b - split) * late
+        cnt = early if b < split else late
+        if b == ranks - 1:
+            cnt = count - off
+        offs.append(off)
+        cnts.append(cnt)
+    return offs, cnts
+
+
+def test_full_allreduce_uneven_segments(pkg, orc, gen, cuda):
+    """The whole compressed ring allreduce of the reference on one GPU, links left out: segmented
+    reduce-scatter with homomorphic sums (HomComp/src/cuda_awareallreduce.cu:456-533), then the
+    all-gather in which every rank decompresses every finished block (:534-565).  The count is
+    not a multiple of anything, so blocks have uneven, unpadded lengths."""
+    torch = cuda
+    orc.set_threads(16)
+    ranks, count = 8, 8 * (1 << 20) + 7777
+    offs, cnts = ring_segments(count, ranks)
+    assert sum(cnts) == count and min(cnts) > 0 and len(set(cnts)) > 1
+    data = [gen.smooth_torch(count, seed=70 + r) for r in range(ranks)]
+    mm = torch.empty(2 * ranks, dtype=torch.float32, device="cuda")
+    with pkg.Workspace(count) as ws:
+        for r in range(ranks):
+            ws.value_range(data[r], mm[2 * r:2 * r + 2])
+    m = mm.cpu().numpy()
+    eb = np.float32(pkg.rel_to_abs(1e-4, float(m[0::2].min()), float(m[1::2].max())))
+    cap = pkg.max_stream_bytes(max(cnts))
+    cur = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    nxt = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    sizes = [0] * ranks
+    results = [torch.zeros(count, dtype=torch.float32, device="cuda") for _ in range(2)]   # two of the ranks' receive buffers
+    with pkg.Workspace(max(cnts)) as ws:
+        for b in range(ranks):   # rank b starts block b
+            ws.compress(data[b][offs[b]:offs[b] + cnts[b]], float(eb), cur[b])
+            sizes[b] = ws.last_size()
+        for k in range(1, ranks):   # block b reaches rank b + k
+            for b in range(ranks):
+                local = data[(b + k) % ranks][offs[b]:offs[b] + cnts[b]]
+                # blocks start at multiples of 4 elements, so the operand stays 16-byte aligned
+                ws.hom_sum_f32(cur[b], sizes[b], local, float(eb), nxt[b])
+                sizes[b] = ws.last_size()
+            cur, nxt = nxt, cur
+        for b in range(ranks):   # all-gather: every rank decompresses the finished block
+            for res in results:
+                ws.decompress(cur[b], sizes[b], cnts[b], float(eb), res[offs[b]:offs[b] + cnts[b]])
+        torch.cuda.synchronize()
+    assert torch.equal(results[0], results[1])
+    got = results[0].cpu().numpy()
+    host = [d.cpu().numpy() for d in data]
+    exact = np.zeros(count, np.float64)
+    for h in host:
+        exact += h
+    assert (np.abs(got.astype(np.float64) - exact) <= ranks * float(eb) * (1 + 1e-3)).all()
+    for b in range(ranks):
+        sl = slice(offs[b], offs[b] + cnts[b])
+        ref = orc.compress(host[b][sl], eb)
+        for k in range(1, ranks):
+            ref = orc.hom_sum_f32(ref, host[(b + k) % ranks][sl], eb)
+        stream = cur[b][:sizes[b]].cpu().numpy()
+        assert stream.size == ref.size and np.array_equal(stream, ref), f"block {b} stream"
+        assert np.array_equal(got[sl].view(np.uint32), orc.decompress(ref, cnts[b], eb).view(np.uint32)), f"block {b} values"
