@@ -182,7 +182,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, ui
     const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
 }
-constexpr int kBufNt = 2;   // cache policy bits of the buffer builtins: non-temporal
+constexpr int kBufNt = 2;   // cache policy bits of the buffer builtins: non-temporal (operands and results, touched once)
+constexpr int kBufCached = 0;   // incoming payload: neighbouring sub-steps share cache lines, so these loads stay cached
 
 // Operand of one sub-step of the tile whose elements start at `tile_elem0` (beyond n: zeros).
 template <int LOCAL>
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         // whole 16-byte pieces; lanes beyond the range get zeros without touching memory
         const __amdgpu_buffer_rsrc_t rs =
             buffer_of(reinterpret_cast<const void *>(ga), tile_of(r) < n_tiles ? (nbytes + 15u) & ~15u : 0u);
-        in[c].chunk = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 0, kBufNt);
+        in[c].chunk = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 0, kBufCached);
     };
     auto request = [&](int64_t r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn]) __attribute__((always_inline)) {
         request_local(r, s, loc);
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                                 buffer_of(reinterpret_cast<const void *>(ga), (nbytes + 15u) & ~15u);
                             for (uint32_t i = (uint32_t)lane + 64u; 16u * i < nbytes; i += 64u)
                                 *reinterpret_cast<u32x4 *>(st + 16u * i) =
-                                    __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(16u * i), 0, kBufNt);
+                                    __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(16u * i), 0, kBufCached);
                         }
                         request_in(c, r2, b2, s2, in);
                         wave_lds_fence();
