@@ -288,6 +288,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     uint32_t hdr_next[kIn];     // header bytes of blocks 2*lane, 2*lane+1 of the next tile
     uint64_t start_next[kIn];   // absolute payload offset of the next tile
     uint64_t start_ctx0[kIn], start_ctx1[kIn];   // of the tiles in the two context buffers (tile parity)
+    // bytes of the stream from the tile's payload start to its stated end, saturated to 32 bits:
+    // everything inside a tile is 32-bit arithmetic against these
+    uint32_t room_ctx0[kIn], room_ctx1[kIn];
     auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             int64_t t = tile_of(r);
@@ -316,7 +319,15 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)hdr_next[c];
                     if ((lane & 7) == 0) s_rel[wave][c][b][lane >> 3] = o0;
                     if (lane == 63) s_rel[wave][c][b][kSub] = incl;
-                    if (b) start_ctx1[c] = start_next[c]; else start_ctx0[c] = start_next[c];
+                    const uint64_t room64 = p.in_size[c] > start_next[c] ? p.in_size[c] - start_next[c] : 0u;
+                    const uint32_t room = room64 > 0xffff0000ull ? 0xffff0000u : (uint32_t)room64;
+                    if (b) {
+                        start_ctx1[c] = start_next[c];
+                        room_ctx1[c] = room;
+                    } else {
+                        start_ctx0[c] = start_next[c];
+                        room_ctx0[c] = room;
+                    }
                 }
                 wave_lds_fence();
             }
@@ -332,16 +343,15 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         rel0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][s]);
         const uint32_t rel1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][s + 1]);
         const uint64_t start = b ? start_ctx1[c] : start_ctx0[c];
-        const uint64_t a = start + rel0;
-        uint64_t e = start + rel1;
         // a block that starts below the stated size is read in full (HomComp/src/GSZ.cu:908-911),
         // nothing further out is touched
-        const uint64_t lim = p.in_size[c] + (kMaxBlockBytes - 1);
-        if (e > lim) e = lim;
-        const uintptr_t g0 = (uintptr_t)p.in[c] + a;
+        const uint32_t room = b ? room_ctx1[c] : room_ctx0[c];
+        const uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
+        const uint32_t end = rel1 < lim ? rel1 : lim;
+        const uintptr_t g0 = (uintptr_t)p.in[c] + start + rel0;
         ga = g0 & ~(uintptr_t)15;
         shift = (uint32_t)(g0 - ga);
-        nbytes = e > a ? shift + (uint32_t)(e - a) : 0u;
+        nbytes = end > rel0 ? shift + (end - rel0) : 0u;
     };
     // The registers of a set are free again as soon as the sub-step has converted the operand /
     // staged the chunk, and the request for the sub-step after the next one is issued right there:
@@ -472,7 +482,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         const uint32_t h = s_hdr_in[wave][c][buf][blk];
                         const uint32_t ofs = s_ofs_in[wave][c][buf][blk];
                         // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
-                        const bool active = size_from_header(h) != 0u && (buf ? start_ctx1[c] : start_ctx0[c]) + ofs < p.in_size[c];
+                        const bool active = size_from_header(h) != 0u && ofs < (buf ? room_ctx1[c] : room_ctx0[c]);
                         int32_t d[8];
                         unpack8(st, shift + ofs - rel0, h, active, k, d);
 #pragma unroll
