@@ -130,7 +130,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; --gpus above 1 is not part of this build "
-              "(the sharding is described in DESIGN.md)", file=sys.stderr)
+              "(chunks are independent: each GPU would run this same path on its share)", file=sys.stderr)
         return 2
 
     import numpy as np
