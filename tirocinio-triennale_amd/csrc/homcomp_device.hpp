@@ -295,20 +295,22 @@ __device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uin
 //
 // The byte offset of a tile's payload in the outgoing stream is an exclusive prefix sum over
 // all earlier tiles (HomComp/src/GSZ.cu:170-239).  It is resolved in a single pass by a division
-// of labour between the data workgroups and one scan-server workgroup of the same launch:
+// of labour between the data waves (one tile per wave and round) and one scan-server workgroup of
+// the same launch:
 //
-//   data workgroup, round i     publishes the tile's byte total in the tile's total word
-//   scan server                 sweeps the total words in tile order, 1024 tiles per step, waits
-//                               until they are all there, scans them and writes every tile's
-//                               exclusive prefix into the tile's prefix word
-//   data workgroup, round i+1   issues the load of the prefix word
-//   data workgroup, round i+2   uses it: the payload goes to its place in the stream
+//   data wave, round i          publishes the tile's byte total in the tile's total word and keeps
+//                               the payload (in LDS, or in its spill area when it does not fit)
+//   scan server                 sweeps the total words in tile order, up to 1024 tiles per step,
+//                               waits until they are all there, scans them and writes every
+//                               tile's exclusive prefix into the tile's prefix word
+//   data wave, round i+D-1      issues the load of the prefix word (D = 2..4 payloads kept)
+//   data wave, round i+D        uses it: the payload goes to its place in the stream
 //
-// so a data workgroup never waits for another data workgroup, only the server waits, and every
-// word is written by one workgroup and read by one.  (Measured on MI355X: read-modify-write
-// atomics on one 128-byte line are serialised at about 11 ns each, and plain loads of a line
-// that is being updated atomically by other compute units are about as slow -- a ticket
-// counter or shared accumulators that thousands of workgroups touch cost more than the codec.)
+// so a data wave never waits for another data wave, only the server waits, and every word is
+// written by one wave and read by one.  (Measured on MI355X: read-modify-write atomics on one
+// 128-byte line are serialised at about 11 ns each, and plain loads of a line that is being
+// updated atomically by other compute units are about as slow -- a ticket counter or shared
+// accumulators that thousands of waves touch cost more than the codec.)
 //
 // A word carries an epoch tag: bits 63-62 state (0 empty, 1 total, 2 exclusive prefix), bits
 // 61-40 the call's epoch, bits 39-0 a byte count; a word of another epoch reads as empty, so the

@@ -42,17 +42,22 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
     if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = stage[head + 16u * nch + tid];
 }
 
-// The scan server: one workgroup of the launch that turns the tile totals the data workgroups
-// publish into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  It sweeps the tiles in index
-// order in steps: wait for the step's totals, scan them, write the prefixes, go on.  The data
-// workgroups publish a whole round (G consecutive tiles) at about the same time, so a step
-// rarely waits long.  Also writes the stream length once the last tile is in.
+// The scan server: one workgroup of the launch that turns the tile totals the data waves publish
+// into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  It sweeps the tiles in index order in
+// steps: wait for the step's totals, scan them, write the prefixes, go on.  The data waves
+// publish a whole round (G consecutive tiles, G = number of data waves) at about the same time,
+// so a step rarely waits long.  Also writes the stream length once the last tile is in.
 //
-// Step size and progress: a data workgroup uses the prefix of its round-r tile in round r+2,
-// before it publishes its round-(r+2) tile.  A step must therefore never contain both a tile and
-// the tile 2G after it (the step could not complete before the workgroup that waits for it has
+// Step size and progress: a data wave uses the prefix of its round-r tile two or more rounds
+// later, before it publishes that round's tile.  A step must therefore never contain both a tile
+// and the tile 2G after it (the step could not complete before the wave that waits for it has
 // published), i.e. a step covers at most 2G tiles: 1024 tiles (4 per lane) when G >= 512,
 // otherwise one tile per lane on min(256, 2G) lanes.
+//
+// Measured on MI355X with per-wave time stamps: on an idle GPU a step takes 0.8 us, next to a
+// full grid of data waves 3.6-3.9 us, whatever the look-ahead of the requests, the number of
+// memory instructions or of waves involved; that pace (about 16 us per round of 4080 tiles)
+// bounds the stream-producing kernels once their own work per round is shorter.
 __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
 {
     __shared__ uint32_t s_wave[kWG / 64];
