@@ -30,6 +30,7 @@ constexpr int kOutBlockBytes = 128;                   // largest payload the enc
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // Every buffer is read or written exactly once per call, so loads and stores carry the
 // non-temporal hint and do not displace the scan words from the caches.

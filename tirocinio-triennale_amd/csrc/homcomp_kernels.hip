@@ -42,6 +42,19 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
     if ((uint32_t)tid < tail) g[head + 16u * nch + tid] = stage[head + 16u * nch + tid];
 }
 
+// Buffer addressing: the descriptor (base, byte count) lives in scalar registers, a lane adds a
+// constant offset, and the hardware checks every dword against the byte count: loads beyond it
+// return 0 and stores beyond it are dropped.  So the ends of the buffers need no branches, a
+// request is a fixed number of memory operations (which lets the compiler wait for exactly the
+// request it needs), and no per-lane address arithmetic is left.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, uint64_t bytes)
+{
+    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+constexpr int kBufNt = 2;   // cache policy bits of the buffer builtins: non-temporal (operands and results, touched once)
+constexpr int kBufCached = 0;   // incoming payload: neighbouring sub-steps share cache lines, so these loads stay cached
+
 // The scan server: one workgroup of the launch that turns the tile totals the data waves publish
 // into exclusive prefixes (HomComp/src/GSZ.cu:170-239).  It sweeps the tiles in index order in
 // steps: wait for the step's totals, scan them, write the prefixes, go on.  The data waves
@@ -54,87 +67,139 @@ __device__ __forceinline__ void copy_out(const uint8_t *stage, uint8_t *g, uint3
 // published), i.e. a step covers at most 2G tiles: 1024 tiles (4 per lane) when G >= 512,
 // otherwise one tile per lane on min(256, 2G) lanes.
 //
-// Measured on MI355X with per-wave time stamps: on an idle GPU a step takes 0.8 us, next to a
-// full grid of data waves 3.6-3.9 us, whatever the look-ahead of the requests, the number of
-// memory instructions or of waves involved; that pace (about 16 us per round of 4080 tiles)
-// bounds the stream-producing kernels once their own work per round is shorter.
-__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
+// Pace: a step is wave-scan arithmetic plus four memory instructions per lane, about 1.2 us next
+// to a full grid of data waves (time stamps of the four server waves), as long as no wait in it
+// covers more than the step's own request: with a wait for all outstanding operations in the
+// look, every step cost a full memory round trip under load (3.7 us) and the server, not the
+// data, set the pace of the stream-producing kernels.
+
+// Status words through buffer addressing: a request or a write-back is a fixed number of memory
+// instructions without a branch around them (lanes beyond the arrays read zeros, their stores
+// are dropped), so the compiler can wait for exactly the request a step needs.  Device scope,
+// like the atomic accesses of the data waves; issue_order() keeps the groups in program order.
+constexpr int kBufStatus = 16;   // sc1
+
+__device__ __forceinline__ void issue_order() { asm volatile("" ::: "memory"); }
+
+template <uint32_t PER>
+__device__ __forceinline__ void scan_server_steps(const TileParams &p, const ScanCtx &c, uint32_t lanes)
 {
-    __shared__ uint32_t s_wave[kWG / 64];
+    __shared__ uint32_t s_wave[2][kWG / 64];   // by step parity: one barrier per step
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const uint32_t per = G >= 512u ? 4u : 1u;                                   // tiles per lane
-    const uint32_t lanes = G >= 512u ? (uint32_t)kWG : (2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
-    const uint32_t step = per * lanes;
+    const uint32_t step = PER * lanes;
+    // lane's place inside a step's words; lanes that take no part point beyond every array
+    const uint32_t voff = (uint32_t)tid < lanes ? (uint32_t)tid * PER * 8u : 0xffffff00u;
     uint64_t base = 0;
+    auto words_from = [&](const uint64_t *arr, uint32_t t0) {
+        // a window from the step's first word; capped below the offset of the lanes that stay out
+        uint64_t left = t0 < c.n_tiles ? (uint64_t)(c.n_tiles - t0) * 8u : 0u;
+        if (left > 0x10000000u) left = 0x10000000u;
+        return buffer_of(arr + (t0 < c.n_tiles ? t0 : 0u), left);
+    };
     // The totals of a step are requested two steps ahead, into two register sets used
     // alternately: in the steady state they were published a round ago, so the server runs at the
-    // pace of its arithmetic instead of one memory round trip per step.  Lanes beyond the end
-    // request the last tiles again (no branch around the loads) and ignore what they get.
-    const uint32_t last = c.n_tiles - per;
-    auto request = [&](uint32_t t0, uint64_t (&dst)[4]) __attribute__((always_inline)) {
-        uint32_t idx = t0 + (uint32_t)tid * per;
-        if (idx > last) idx = last;
-        dst[0] = status_load(&c.totals[idx]);
-        if (per == 4u) {
-            dst[1] = status_load(&c.totals[idx + 1]);
-            dst[2] = status_load(&c.totals[idx + 2]);
-            dst[3] = status_load(&c.totals[idx + 3]);
-        }
-    };
-    auto process = [&](uint32_t t0, uint64_t (&w)[4]) __attribute__((always_inline)) {
-        const uint32_t idx = t0 + (uint32_t)tid * per;   // with per == 4: n_tiles is a multiple of 8
-        const bool in = (uint32_t)tid < lanes && idx < c.n_tiles;
-        if (in) {
-            uint32_t spins = 0;
-            for (;;) {
-                bool ok = status_state(w[0], c.epoch) == 1u;
-                if (per == 4u)
-                    ok = ok && status_state(w[1], c.epoch) == 1u && status_state(w[2], c.epoch) == 1u &&
-                         status_state(w[3], c.epoch) == 1u;
-                if (ok || scan_give_up(c, spins)) break;
-                request(t0, w);
+    // pace of its arithmetic instead of one memory round trip per step.
+    auto request = [&](uint32_t t0, uint64_t (&dst)[PER]) __attribute__((always_inline)) {
+        const __amdgpu_buffer_rsrc_t rs = words_from(c.totals, t0);
+        if constexpr (PER == 4) {   // two words per instruction: the step's cost is its memory instructions
+            const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, 0, kBufStatus);
+            const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(voff + 16u), 0, kBufStatus);
+            dst[0] = ((uint64_t)a.y << 32) | a.x; dst[1] = ((uint64_t)a.w << 32) | a.z;
+            dst[2] = ((uint64_t)b.y << 32) | b.x; dst[3] = ((uint64_t)b.w << 32) | b.z;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j) {
+                const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)(voff + 8u * j), 0, kBufStatus);
+                dst[j] = ((uint64_t)w.y << 32) | w.x;
             }
         }
-        uint32_t v[4], mine = 0;
+        issue_order();
+    };
+    auto process = [&](uint32_t t0, uint32_t parity, uint64_t (&w)[PER]) __attribute__((always_inline)) {
+        const uint32_t idx = t0 + (uint32_t)tid * PER;   // n_tiles is a multiple of PER when PER > 1
+        const bool in = (uint32_t)tid < lanes && t0 < c.n_tiles && idx < c.n_tiles;   // t0 beyond the end: an empty step
+        auto all_there = [&]() {
+            uint32_t ok = 1u;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            v[j] = in && j < per ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+            for (uint32_t j = 0; j < PER; ++j) ok &= (uint32_t)(status_state(w[j], c.epoch) == 1u);
+            return ok != 0u;
+        };
+        // The first look is straight-line code, for every lane: the wait in front of it covers
+        // this step's request only and leaves the later requests and the write-backs in flight.
+        // (A look inside a retry loop, or behind a branch, makes the compiler wait for every
+        // outstanding operation, the newest request included: a memory round trip per step.)
+        const bool there = all_there();
+        if (in && !there) {
+            uint32_t spins = 0;
+            do {
+                if (scan_give_up(c, spins)) break;
+                uint64_t again[PER];
+#pragma unroll
+                for (uint32_t j = 0; j < PER; ++j) again[j] = status_load(&c.totals[idx + j]);
+#pragma unroll
+                for (uint32_t j = 0; j < PER; ++j) w[j] = again[j];
+            } while (!all_there());
+        }
+        uint32_t v[PER], mine = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < PER; ++j) {
+            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
             mine += v[j];
         }
         const uint32_t incl = wave_incl_scan_u32(mine, lane);
-        if (lane == 63) s_wave[wave] = incl;
+        if (lane == 63) s_wave[parity][wave] = incl;
         __syncthreads();
         uint32_t before = 0, step_total = 0;
 #pragma unroll
         for (int q = 0; q < kWG / 64; ++q) {
-            const uint32_t t = s_wave[q];
+            const uint32_t t = s_wave[parity][q];
             if (q < wave) before += t;
             step_total += t;
         }
-        if (in) {
-            uint64_t run = base + before + (incl - mine);
+        const __amdgpu_buffer_rsrc_t rp = words_from(c.prefixes, t0);
+        uint64_t run = base + before + (incl - mine);
+        uint64_t o[PER];
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                if (j < per) {
-                    status_store(&c.prefixes[idx + j], status_word(c.epoch, 2, run));
-                    run += v[j];
-                }
-            }
+        for (uint32_t j = 0; j < PER; ++j) {
+            o[j] = status_word(c.epoch, 2, run);
+            run += v[j];
         }
+        if constexpr (PER == 4) {
+            __builtin_amdgcn_raw_buffer_store_b128(
+                u32x4{(uint32_t)o[0], (uint32_t)(o[0] >> 32), (uint32_t)o[1], (uint32_t)(o[1] >> 32)}, rp, (int)voff, 0, kBufStatus);
+            __builtin_amdgcn_raw_buffer_store_b128(
+                u32x4{(uint32_t)o[2], (uint32_t)(o[2] >> 32), (uint32_t)o[3], (uint32_t)(o[3] >> 32)}, rp, (int)(voff + 16u), 0,
+                kBufStatus);
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j)
+                __builtin_amdgcn_raw_buffer_store_b64(u32x2{(uint32_t)o[j], (uint32_t)(o[j] >> 32)}, rp, (int)(voff + 8u * j), 0,
+                                                      kBufStatus);
+        }
+        issue_order();
         base += step_total;
-        __syncthreads();   // s_wave is reused by the next step
     };
-    uint64_t wa[4] = {0, 0, 0, 0}, wb[4] = {0, 0, 0, 0};
+    // One loop shape for filling the pipeline and for the steady state: the first pass processes
+    // two empty steps (a window beyond the end: no lane takes part) and issues the first two
+    // requests.  Every path into a look then carries the same number of later operations, which
+    // is what lets the compiler count instead of waiting for all of them.
+    uint64_t wa[PER], wb[PER];
+#pragma unroll
+    for (uint32_t j = 0; j < PER; ++j) wa[j] = wb[j] = 0;
+    const uint32_t none = 0xffffffffu;
+    const uint64_t end = (uint64_t)c.n_tiles;
+    process(none, 0, wa);
     request(0, wa);
+    process(none, 1, wb);
     request(step, wb);
-    for (uint32_t t0 = 0; t0 < c.n_tiles; t0 += 2 * step) {
-        process(t0, wa);
-        request(t0 + 2 * step, wa);
-        if (t0 + step >= c.n_tiles) break;
-        process(t0 + step, wb);
-        request(t0 + 3 * step, wb);
+    for (uint64_t t0 = 0; t0 < end; t0 += 2ull * step) {
+        auto at = [&](uint64_t t) { return t < end ? (uint32_t)t : none; };
+        process(at(t0), 0, wa);
+        request(at(t0 + 2ull * step), wa);
+        process(at(t0 + step), 1, wb);
+        request(at(t0 + 3ull * step), wb);
     }
     if (tid == 0) {
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
@@ -143,6 +208,14 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
         // mean payload bytes per tile, for the host's choice of the next launch's LDS budget
         if (p.host_total) *p.host_total = base / c.n_tiles;
     }
+}
+
+__device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &c, uint32_t G)
+{
+    if (G >= 512u)
+        scan_server_steps<4>(p, c, (uint32_t)kWG);
+    else
+        scan_server_steps<1>(p, c, 2u * G < (uint32_t)kWG ? 2u * G : (uint32_t)kWG);
 }
 
 // ---------------------------------------------------------------- wave-autonomous kernels
@@ -176,19 +249,6 @@ struct SubRegs {
     f32x4 f[2];
     i32x4 i[2];
 };
-
-// Buffer addressing: the descriptor (base, byte count) lives in scalar registers, a lane adds a
-// constant offset, and the hardware checks every dword against the byte count: loads beyond it
-// return 0 and stores beyond it are dropped.  So the ends of the buffers need no branches, a
-// request is a fixed number of memory operations (which lets the compiler wait for exactly the
-// request it needs), and no per-lane address arithmetic is left.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, uint64_t bytes)
-{
-    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
-}
-constexpr int kBufNt = 2;   // cache policy bits of the buffer builtins: non-temporal (operands and results, touched once)
-constexpr int kBufCached = 0;   // incoming payload: neighbouring sub-steps share cache lines, so these loads stay cached
 
 // Operand of one sub-step of the tile whose elements start at `tile_elem0` (beyond n: zeros).
 template <int LOCAL>
@@ -421,6 +481,19 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                 // the prefix word travels in lane 0 only: a device-scope load is executed per
                 // lane, so 64 lanes asking for the same word would be 64 requests
                 uint64_t excl = 0;
+                {
+                    // Every wave of a round has to publish before the round's last prefixes
+                    // exist, so the launch moves at the pace of its slowest waves (the hardware
+                    // favours the oldest waves of a SIMD: the workgroup that arrived last on a
+                    // compute unit ran 60 % slower per tile than the first).  A wave whose
+                    // prefix is already there runs behind the scan and takes the higher issue
+                    // priority for this round; one that has to wait runs ahead and yields.
+                    const int behind = __builtin_amdgcn_readfirstlane((int)(status_state(probe, scan.epoch) == 2u));
+                    if (behind)
+                        __builtin_amdgcn_s_setprio(1);
+                    else
+                        __builtin_amdgcn_s_setprio(0);
+                }
                 if (lane == 0) excl = scan_resolve(scan, (uint32_t)td, probe);
                 excl = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(excl >> 32)) << 32) |
                        (uint32_t)__builtin_amdgcn_readfirstlane((int)excl);
