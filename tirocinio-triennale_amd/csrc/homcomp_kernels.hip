@@ -323,7 +323,8 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // the launch (dynamic LDS), see TileParams
     extern __shared__ __align__(16) uint8_t s_dyn[];
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
-    __shared__ __align__(16) uint8_t s_in[kW][kIn][NIN > 0 ? kInStage : 16];
+    // one stage per wave: the incoming streams of a sub-step are decoded one after the other
+    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInStage : 16];
     __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
     __shared__ __align__(4) uint8_t s_hdr_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 4];
     __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512];     // decoder: exchange of the lanes' output pieces
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         uintptr_t ga;
                         uint32_t shift, nbytes, rel0;
                         range_of(c, buf, s, ga, shift, nbytes, rel0);
-                        uint8_t *st = s_in[wave][c];
+                        uint8_t *st = s_in[wave];
                         if (16u * (uint32_t)lane < nbytes)
                             *reinterpret_cast<u32x4 *>(st + 16u * lane) = in[c].chunk;
                         if (nbytes > 1024u) {   // a range of more than 64 pieces: the rest is fetched now
@@ -565,7 +566,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         unpack8(st, shift + ofs - rel0, h, active, k, d);
 #pragma unroll
                         for (int m = 0; m < 8; ++m) v[m] = (int32_t)((uint32_t)v[m] + (uint32_t)d[m]);
-                        wave_lds_fence();   // the stage is rewritten by the next sub-step
+                        wave_lds_fence();   // the stage is rewritten by the next stream and the next sub-step
                     }
                 }
                 if constexpr (!kEnc) {
@@ -584,12 +585,17 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     // The lanes' 32-byte pieces are exchanged through LDS so that each store
                     // instruction writes 1 KiB of consecutive bytes (full cache lines): stores of
                     // 16 bytes at a 32-byte stride reach only a fraction of the write bandwidth.
+                    // 16-byte piece P of the 2 KiB lives at piece P ^ x(P), x = bit 3 ^ bit 4 of P:
+                    // a lane writes pieces 2 * lane and 2 * lane + 1 and reads pieces lane and
+                    // 64 + lane, and with the swap the lanes that access the LDS in the same
+                    // cycle (8 or 16 neighbours) hit different banks both ways.
                     float *tr = s_tr[wave];
-                    *reinterpret_cast<f32x4 *>(tr + 8 * lane) = f32x4{y[0], y[1], y[2], y[3]};
-                    *reinterpret_cast<f32x4 *>(tr + 8 * lane + 4) = f32x4{y[4], y[5], y[6], y[7]};
+                    const int xw = ((lane >> 2) ^ (lane >> 3)) & 1, xr = ((lane >> 3) ^ (lane >> 4)) & 1;
+                    *reinterpret_cast<f32x4 *>(tr + 4 * (2 * lane + xw)) = f32x4{y[0], y[1], y[2], y[3]};
+                    *reinterpret_cast<f32x4 *>(tr + 4 * (2 * lane + 1 - xw)) = f32x4{y[4], y[5], y[6], y[7]};
                     wave_lds_fence();
-                    const f32x4 lo = *reinterpret_cast<const f32x4 *>(tr + 4 * lane);
-                    const f32x4 hi = *reinterpret_cast<const f32x4 *>(tr + 256 + 4 * lane);
+                    const f32x4 lo = *reinterpret_cast<const f32x4 *>(tr + 4 * (lane ^ xr));
+                    const f32x4 hi = *reinterpret_cast<const f32x4 *>(tr + 256 + 4 * (lane ^ xr));
                     wave_lds_fence();
                     const __amdgpu_buffer_rsrc_t ro =
                         buffer_of(p.out_f32 + tile_elem0, tile_elem0 < p.n ? (p.n - tile_elem0) * 4u : 0u);
