@@ -880,7 +880,22 @@ static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
     const void *fn = reinterpret_cast<const void *>(&k_wave<NIN, LOCAL, OUT>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
     if (e != hipSuccess) return e;
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, dyn);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, dyn);
+    // The stream-producing kernels need every workgroup of the grid resident at the same time
+    // (the scan's waits).  Near the LDS limit the runtime's answer was one workgroup too many on
+    // MI355X (5 x 32 688 bytes reported to fit 160 KiB; the fifth was not resident and the waits
+    // ran into their bound), so the grid stays within what a 2 KiB allocation unit leaves room
+    // for and within four workgroups per compute unit.
+    if (e == hipSuccess && OUT == kOutStream) {
+        hipFuncAttributes fa;
+        e = hipFuncGetAttributes(&fa, fn);
+        if (e != hipSuccess) return e;
+        const size_t unit = 2048, per_wg = (fa.sharedSizeBytes + dyn + unit - 1) / unit * unit;
+        const int by_lds = (int)((160u * 1024u - unit) / per_wg);
+        if (*blocks_per_cu > by_lds) *blocks_per_cu = by_lds;
+        if (*blocks_per_cu > 4) *blocks_per_cu = 4;
+    }
+    return e;
 }
 
 hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu)
