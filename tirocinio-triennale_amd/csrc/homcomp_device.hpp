@@ -93,6 +93,17 @@ __device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t x, int /*lane*/)
     return x;
 }
 
+// The same for a value that is equal in the four lanes of every quad: the inclusive sum over the
+// quads up to the lane's own, with two row shifts less.
+__device__ __forceinline__ uint32_t quad_incl_scan_u32(uint32_t x)
+{
+    x += dpp_u32<0x114>(x);   // row_shr:4
+    x += dpp_u32<0x118>(x);   // row_shr:8
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xA, 0xF, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xC, 0xF, false);
+    return x;
+}
+
 // ---------------------------------------------------------------- scalar arithmetic
 
 // HomComp/src/GSZ.cu:6-25: fl(x*r), compare with -0.5, fl(.+0.5), convert toward zero
@@ -267,8 +278,9 @@ __device__ __forceinline__ void unpack_group(const uint8_t *stage, uint32_t base
     }
 }
 
-__device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uint32_t hdr,
-                                        bool active, int k, int32_t v[8])
+// Decodes the lane's eight deltas of a block and adds them to v[] (wrapping).
+__device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0, uint32_t hdr,
+                                            bool active, int k, int32_t v[8])
 {
     if (!active) hdr = 0;
     const uint32_t sel = hdr >> 7;
@@ -288,7 +300,8 @@ __device__ __forceinline__ void unpack8(const uint8_t *stage, uint32_t pos0, uin
 #pragma unroll
     for (int m = 0; m < 8; ++m) {                         // :1432-1434
         const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)sb, 7 - m, 1);   // 0 or ~0
-        v[m] = (int32_t)((a[m] ^ mask) - mask);
+        // v + ((a ^ mask) - mask), in the order that is one xor-add
+        v[m] = (int32_t)((a[m] ^ mask) + ((uint32_t)v[m] - mask));
     }
 }
 

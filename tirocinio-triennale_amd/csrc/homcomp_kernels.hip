@@ -562,10 +562,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         const uint32_t ofs = s_ofs_in[wave][c][buf][blk];
                         // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
                         const bool active = size_from_header(h) != 0u && ofs < (buf ? room_ctx1[c] : room_ctx0[c]);
-                        int32_t d[8];
-                        unpack8(st, shift + ofs - rel0, h, active, k, d);
-#pragma unroll
-                        for (int m = 0; m < 8; ++m) v[m] = (int32_t)((uint32_t)v[m] + (uint32_t)d[m]);
+                        unpack8_add(st, shift + ofs - rel0, h, active, k, v);
                         wave_lds_fence();   // the stage is rewritten by the next stream and the next sub-step
                     }
                 }
@@ -603,11 +600,11 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, hi), ro, lane * 16 + 1024, s * 2048, kBufNt);
                 } else {
                     // ---- rate selection (HomComp/src/GSZ.cu:151-167) and the block's offset: the
-                    //      sizes are equal in the four lanes of a quad, so a wave scan of the first
-                    //      lanes' values minus the own size is the exclusive prefix in every lane
+                    //      sizes are equal in the four lanes of a quad, so a scan over the quads
+                    //      minus the own size is the exclusive prefix in every lane
                     uint32_t a[8], sb, hd, size, a0;
                     analyse8(v, k, a, sb, hd, size, a0);
-                    const uint32_t incl = wave_incl_scan_u32(k == 0 ? size : 0u, lane);
+                    const uint32_t incl = quad_incl_scan_u32(size);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     const uint32_t pos = run + incl - size;
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
