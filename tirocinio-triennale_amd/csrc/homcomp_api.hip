@@ -110,10 +110,12 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 
 // LDS stage per data wave (two deferred tiles by default).  The small budgets fit tiles of streams
 // compressed about 4x or better and let more waves share a compute unit; the large one holds
-// tiles down to a ratio of 2.  A tile beyond its slot still works (it goes through the spill
-// area), only slower, so the choice below is a performance heuristic, never a correctness matter.
+// tiles down to a ratio of 2 (2.1 with two incoming streams, whose kernel holds more LDS of its
+// own: with the full 8 KiB slots only one of its workgroups fits a compute unit, and that is
+// slower than spilling).  A tile beyond its slot still works (it goes through the spill area),
+// only slower, so the choice below is a performance heuristic, never a correctness matter.
 constexpr uint32_t kStageSmall[hc::kOpCount] = {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)};
-constexpr uint32_t kStageLarge = 2 * (8192 + 64);
+constexpr uint32_t kStageLarge[hc::kOpCount] = {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7680 + 64)};
 
 // expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
@@ -130,7 +132,7 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         if (ws->stage_class >= 0) cls = ws->stage_class;
         p.host_total = &ws->h_mean_tile[op];
     }
-    p.stage_bytes = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge : kStageSmall[op]);
+    p.stage_bytes = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge[op] : kStageSmall[op]);
     return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -222,7 +224,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     for (int op = 0; ok && op < hc::kOpCount; ++op) {
         for (int cls = 0; ok && cls < 2; ++cls) {
             int per_cu = 0;
-            const uint32_t stage = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge : kStageSmall[op]);
+            const uint32_t stage = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge[op] : kStageSmall[op]);
             ok = hip_ok(hc::op_kernel_residency(op, stage, &per_cu));
             if (ok && per_cu < 1) per_cu = 1;
             // one compute unit's worth of workgroups is left free: the persistent grid must be fully
