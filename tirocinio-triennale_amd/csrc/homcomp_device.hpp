@@ -142,6 +142,18 @@ __device__ __forceinline__ uint32_t size_from_header(uint32_t h)
     return (h & 0x80u) ? 4u + 4u * F + ob : (F ? 4u + 4u * F : 0u);
 }
 
+// The same for four header bytes at once, added to acc: byte-parallel arithmetic (a size is at
+// most 132, so nothing carries from byte to byte) and one sum-of-bytes instruction.
+__device__ __forceinline__ uint32_t add_sizes_from_4_headers(uint32_t w, uint32_t acc)
+{
+    const uint32_t F = w & 0x1f1f1f1fu;
+    const uint32_t sel = (w >> 7) & 0x01010101u;
+    const uint32_t has_planes = ((F + 0x7f7f7f7fu) >> 7) & 0x01010101u;   // F != 0
+    const uint32_t ob = (((w >> 5) & 0x03030303u) + 0x01010101u) & (sel * 0xffu);
+    const uint32_t sizes = (F << 2) + ((has_planes | sel) << 2) + ob;
+    return __builtin_amdgcn_sad_u8(sizes, 0u, acc);
+}
+
 // Transpose of an 8x8 bit matrix held row-per-byte in (lo, hi): result bit (8r+c) = input bit
 // (8c+r).  Three rounds of delta swaps; the first two stay inside the 32-bit halves, only the last
 // one moves nibbles between them, so everything is full-rate 32-bit arithmetic.

@@ -683,30 +683,42 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
     uint32_t acc = 0;
     constexpr uint32_t kPieces = kTileBlocks / 16;            // 16-byte header pieces (lanes) per tile
     constexpr uint32_t kPasses = kOfsBlockTiles * kPieces / 256;
+    // all pieces of the thread are requested before the first is used: the kernel is a handful of
+    // dependent memory round trips otherwise (9 us for any stream length)
+    u32x4 q[kPasses];
+    const bool aligned = ((uintptr_t)hdr & 15u) == 0;
+#pragma unroll
     for (uint32_t it = 0; it < kPasses; ++it) {
         const uint32_t t = (blockIdx.x * kPasses + it) * 256u + threadIdx.x;   // piece index
-        const uint32_t tile = t / kPieces;
-        uint32_t sum = 0;
-        if (tile < n_tiles) {
+        q[it] = u32x4{0u, 0u, 0u, 0u};   // zero header bytes: blocks of size 0
+        if (t / kPieces < n_tiles) {
             const uint8_t *src = hdr + (uint64_t)t * 16u;
-            uint32_t w[4];
-            if (((uintptr_t)src & 15u) == 0) {
-                const u32x4 q = *reinterpret_cast<const u32x4 *>(src);
-                w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+            if (aligned) {
+                q[it] = *reinterpret_cast<const u32x4 *>(src);
             } else {
+                uint32_t w[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     w[i] = (uint32_t)src[4 * i] | ((uint32_t)src[4 * i + 1] << 8) |
                            ((uint32_t)src[4 * i + 2] << 16) | ((uint32_t)src[4 * i + 3] << 24);
+                q[it] = u32x4{w[0], w[1], w[2], w[3]};
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int b = 0; b < 4; ++b) sum += size_from_header((w[i] >> (8 * b)) & 0xffu);
         }
-        acc += sum;
+    }
 #pragma unroll
-        for (uint32_t d = 1; d < kPieces; d <<= 1) sum += __shfl_xor(sum, d, 64);
+    for (uint32_t it = 0; it < kPasses; ++it) {
+        const uint32_t t = (blockIdx.x * kPasses + it) * 256u + threadIdx.x;
+        const uint32_t tile = t / kPieces;
+        uint32_t sum = add_sizes_from_4_headers(q[it].x, 0u);
+        sum = add_sizes_from_4_headers(q[it].y, sum);
+        sum = add_sizes_from_4_headers(q[it].z, sum);
+        sum = add_sizes_from_4_headers(q[it].w, sum);
+        acc += sum;
+        // the eight pieces of a tile sit in eight neighbouring lanes
+        static_assert(kPieces == 8, "reduction over groups of eight lanes");
+        sum += dpp_u32<kDppXor1>(sum);
+        sum += dpp_u32<kDppXor2>(sum);
+        sum += dpp_u32<kDppRowHalfMirror>(sum);   // the other quad of the eight
         if (tile < n_tiles && (threadIdx.x & (kPieces - 1)) == 0) totals[tile] = sum;
     }
     const uint32_t block_total = wg_reduce_u32(acc, s_tmp);
