@@ -334,3 +334,34 @@ def test_lds_budget_follows_the_data(pkg, cuda, orc, gen):
             assert_stream_equal(g.compress(x, np.float32(eb)), orc.compress(x, np.float32(eb)), f"compress #{seed}")
     finally:
         g.close()
+
+
+def test_two_streams_do_not_overlap_their_scans(pkg, cuda, orc, gen):
+    """Two workspaces driven from two streams at the same time.  Every stream-producing kernel
+    needs its whole grid resident, so the library orders such launches across the streams of a
+    process; interleaved calls must give the oracle's bytes and no scan time-out."""
+    torch = cuda
+    orc.set_threads(16)
+    n = 1 << 24                      # 4096 tiles: each launch asks for the full persistent grid
+    eb = np.float32(8e-4)
+    a, b = gen.smooth_np(n, 61), gen.smooth_np(n, 62)
+    want_a, want_b = orc.compress(a, eb), orc.compress(b, eb)
+    want_sum = orc.hom_sum_f32(want_a, b, eb)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    cap = pkg.max_stream_bytes(n)
+    out1 = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    out2 = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    sa = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    sa[:want_a.size] = torch.from_numpy(want_a).cuda()
+    torch.cuda.synchronize()
+    with pkg.Workspace(n) as w1, pkg.Workspace(n) as w2:
+        for i in range(12):
+            w1.compress(da if i % 2 == 0 else db, float(eb), out1[i % 2], stream=s1)
+            w2.hom_sum_f32(sa, want_a.size, db, float(eb), out2[i % 2], stream=s2)
+        L1, L2 = w1.last_size(stream=s1), w2.last_size(stream=s2)
+        torch.cuda.synchronize()
+        assert L1 == want_b.size and L2 == want_sum.size
+        assert_stream_equal(out1[1][:L1].cpu().numpy(), want_b, "compress on stream 1")
+        assert_stream_equal(out1[0][:want_a.size].cpu().numpy(), want_a, "compress on stream 1 (even calls)")
+        assert_stream_equal(out2[1][:L2].cpu().numpy(), want_sum, "hom_sum_f32 on stream 2")

@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "homcomp_kernels.hpp"
@@ -117,6 +118,48 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 constexpr uint32_t kStageSmall[hc::kOpCount] = {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)};
 constexpr uint32_t kStageLarge[hc::kOpCount] = {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7680 + 64)};
 
+// The stream-producing kernels of this process never overlap on a device.  Each of them needs
+// its whole grid resident (the scan's waits), and two such grids from different streams can each
+// end up half resident, every wave waiting for workgroups that cannot start: both calls would
+// run into the bound of their waits.  So a launch on another stream than the device's previous
+// one first waits (on the GPU, not on the host) for an event recorded on that stream.  A stream under capture is
+// left alone: its graph orders the launches it contains.
+struct DeviceChain {
+    std::mutex mu;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool any = false;
+};
+DeviceChain g_chain[64];
+
+int chained_launch(homcomp_workspace *ws, int op, const hc::TileParams &p, uint32_t max_grid, hipStream_t s)
+{
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+    if (capturing || ws->device < 0 || ws->device >= 64) {
+        if (capturing) (void)hipGetLastError();
+        return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    }
+    DeviceChain &c = g_chain[ws->device];
+    std::lock_guard<std::mutex> lock(c.mu);
+    if (c.any && c.last != s) {
+        // The event is recorded only now, on the stream of the previous launch (a call that stays
+        // on one stream pays nothing): it covers that launch and whatever followed it there.
+        if (!c.done && !hip_ok(hipEventCreateWithFlags(&c.done, hipEventDisableTiming))) return HOMCOMP_ERR_HIP;
+        if (hipEventRecord(c.done, c.last) == hipSuccess) {
+            if (!hip_ok(hipStreamWaitEvent(s, c.done, 0))) return HOMCOMP_ERR_HIP;
+        } else {
+            // the previous stream is gone: wait for the device instead
+            (void)hipGetLastError();
+            if (!hip_ok(hipDeviceSynchronize())) return HOMCOMP_ERR_HIP;
+        }
+    }
+    if (!hip_ok(hc::launch_op(op, p, max_grid, s))) return HOMCOMP_ERR_HIP;
+    c.last = s;
+    c.any = true;
+    return HOMCOMP_OK;
+}
+
 // expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
@@ -133,7 +176,8 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         p.host_total = &ws->h_mean_tile[op];
     }
     p.stage_bytes = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge[op] : kStageSmall[op]);
-    return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    if (op == hc::kOpDecompress) return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    return chained_launch(ws, op, p, ws->max_grid[op][cls], s);
 }
 
 // payload bytes per tile of an incoming stream
