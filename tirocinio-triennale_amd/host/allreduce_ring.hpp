@@ -19,6 +19,9 @@
 //     more than the stream); the true stream length is sent;
 //   * the padding of the temporary array is zero-filled (the reference reduces whatever
 //     cudaMalloc left there; it is never copied out);
+//   * where the padding of the segmented variants pushes the start of the last block beyond
+//     the array (count far below its multiple of 32768) the reference's block count goes
+//     negative; here that block is empty and the blocks before it carry the padding;
 //   * buffers and the workspace can be kept between calls (RingBuffers), which is what the
 //     reference's _opt variant does by hand (:745-760).
 // Returns 0, or the first non-zero status (HOMCOMP_ERR_* or the communicator's).
