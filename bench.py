@@ -112,6 +112,33 @@ def sweep(torch, pkg, gen) -> int:
     return 0
 
 
+def error_measures(torch, x, y, dec, eb, chunk=1 << 24):
+    """Maximum absolute error, PSNR, NRMSE and correlation of dec against the exact x + y (float64),
+    accumulated chunk by chunk on the GPU; two operands, so the bound is 2 * eb."""
+    n = x.numel()
+    lo, hi, dmax = float("inf"), float("-inf"), 0.0
+    s_o = s_d = s_oo = s_dd = s_od = s_ee = 0.0
+    for i in range(0, n, chunk):
+        o = x[i:i + chunk].double() + y[i:i + chunk].double()
+        d = dec[i:i + chunk].double()
+        e = d - o
+        lo, hi = min(lo, float(o.min())), max(hi, float(o.max()))
+        dmax = max(dmax, float(e.abs().max()))
+        s_o += float(o.sum()); s_d += float(d.sum())
+        s_oo += float((o * o).sum()); s_dd += float((d * d).sum()); s_od += float((o * d).sum())
+        s_ee += float((e * e).sum())
+    mse, rng = s_ee / n, hi - lo
+    cov = s_od / n - (s_o / n) * (s_d / n)
+    var_o, var_d = s_oo / n - (s_o / n) ** 2, s_dd / n - (s_d / n) ** 2
+    import math
+    # the reference quantises and dequantises in float32: each operand may exceed eb by 2^-21 of its
+    # magnitude, which the 0.1 % of slack covers for these inputs (the parity tests use the same)
+    return {"max_abs_err": dmax, "bound": 2 * eb, "within_bound": bool(dmax <= 2 * eb * (1 + 1e-3)),
+            "psnr_db": round(20 * math.log10(rng) - 10 * math.log10(mse), 3) if mse > 0 and rng > 0 else None,
+            "nrmse": math.sqrt(mse) / rng if rng > 0 else None,
+            "correlation": round(cov / math.sqrt(var_o * var_d), 9) if var_o > 0 and var_d > 0 else None}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -226,6 +253,13 @@ def main() -> int:
         "ops": ops,
         "roofline": roofline,
     }
+
+    # Reconstruction quality of the reduced values, with the measures of the reference's evaluator
+    # (HomComp/src/homcomp_eval.cu:72-133): decompress(hom_sum(compress(x), y)) against x + y.
+    ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s)
+    ws.decompress(cmp_s, ls, n, eb, dec)
+    torch.cuda.synchronize()
+    out["error"] = error_measures(torch, x, y, dec, eb)
 
     if not args.no_cpu:
         orc = entry.load_oracle()
