@@ -2,7 +2,9 @@
 // R ranks as host threads on one GPU (loopback_comm.hpp), the way the reference's benchmark drives
 // them over MPI (HomComp/src/cuda_awareallreduce.cu).
 //   ring_allreduce <F|I|Fseg|Iseg|Fopt> <ranks> <count> <eb> <in_prefix> <out_prefix> [repeats]
-// reads <in_prefix>.r<k>.f32 (count floats per rank), writes <out_prefix>.r<k>.f32, prints status=<rc>.
+// reads <in_prefix>.r<k>.f32 (count floats per rank), writes <out_prefix>.r<k>.f32, prints status=<rc> and
+// the wall time per call of rank 0 (calls after the first, which allocates).
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <string>
@@ -45,6 +47,8 @@ int main(int argc, char **argv)
 
     homcomp::LoopbackWorld world(ranks);
     std::vector<int> status((size_t)ranks, -1);
+    std::chrono::steady_clock::time_point t_second;
+    double ms_per_call = 0.0;
     std::vector<std::thread> threads;
     for (int r = 0; r < ranks; ++r) {
         threads.emplace_back([&, r] {
@@ -58,13 +62,20 @@ int main(int argc, char **argv)
             if (!rc && hipMemcpy(d_sbuf, host.data(), count * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) rc = 102;
             // a rank that failed before the ring still has to take part in it, or the others would wait
             homcomp::RingComm &comm = world.comm(r);
+            const auto t_begin = std::chrono::steady_clock::now();
             for (int it = 0; it < repeats && !rc; ++it) {
+                if (it == 1 && r == 0) t_second = std::chrono::steady_clock::now();   // the first call allocates
                 if (variant == "F") rc = allreduce_ring_comprs_hom_sum_F(d_sbuf, d_rbuf, count, comm, eb);
                 else if (variant == "I") rc = allreduce_ring_comprs_hom_sum(d_sbuf, d_rbuf, count, comm, eb);
                 else if (variant == "Fseg") rc = allreduce_ring_comprs_hom_sum_F_seg(d_sbuf, d_rbuf, count, comm, eb);
                 else if (variant == "Iseg") rc = allreduce_ring_comprs_hom_sum_seg(d_sbuf, d_rbuf, count, comm, eb);
                 else if (variant == "Fopt") rc = allreduce_ring_comprs_hom_sum_F_opt(d_sbuf, d_rbuf, count, comm, eb);
                 else rc = 2;
+            }
+            if (r == 0) {
+                const auto t_end = std::chrono::steady_clock::now();
+                const auto from = repeats > 1 ? t_second : t_begin;
+                ms_per_call = std::chrono::duration<double, std::milli>(t_end - from).count() / (repeats > 1 ? repeats - 1 : 1);
             }
             if (!rc && hipMemcpy(host.data(), d_rbuf, count * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) rc = 103;
             if (!rc && !write_file(out + ".r" + std::to_string(r) + ".f32", host)) rc = 104;
@@ -77,6 +88,6 @@ int main(int argc, char **argv)
     int worst = 0;
     for (int rc : status)
         if (rc != 0) worst = rc;
-    std::printf("status=%d\n", worst);
+    std::printf("status=%d ms_per_call=%.3f\n", worst, ms_per_call);
     return worst == 0 ? 0 : 1;
 }
