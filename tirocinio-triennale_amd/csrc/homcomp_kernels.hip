@@ -454,6 +454,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // r + D - 1 and used at the start of round r + D.  The wave's LDS stage is cut into D slots;
     // more, smaller slots give the scan more time to come back (the words travel through memory,
     // several microseconds each way under load) at the price of spilling tiles beyond a slot.
+    // Measured on MI355X: two slots are enough, three or four are not faster.
     const int D = (int)p.out_slots;
     const uint32_t slot_bytes = (p.stage_bytes / (uint32_t)D) & ~15u;
     const uint32_t slot_cap = slot_bytes - 64u;
