@@ -193,3 +193,42 @@ def test_full_allreduce_uneven_segments(pkg, orc, gen, cuda):
         stream = cur[b][:sizes[b]].cpu().numpy()
         assert stream.size == ref.size and np.array_equal(stream, ref), f"block {b} stream"
         assert np.array_equal(got[sl].view(np.uint32), orc.decompress(ref, cnts[b], eb).view(np.uint32)), f"block {b} values"
+
+
+def test_stream_longer_than_4_gib(pkg, cuda):
+    """Maximum sizes: 2^30 + 12345 incompressible values give a stream of 4.3e9 bytes, beyond the
+    32-bit offsets of the reference (HomComp/src/GSZ.cu:170-239 keeps them in unsigned int); the
+    offsets here are 64-bit.  No CPU pass at this size: the checks are properties of the codec.
+    Values are multiples of 64 below 2^30 with eb = 0.5: the quantised values survive the trip
+    through float32 (the reference's two float roundings move negative values by one, which float32
+    holds or rounds back), so compress(decompress(s)) must give s back byte for byte."""
+    torch = cuda
+    n = (1 << 30) + 12345
+    x = torch.randint(-(1 << 24) + 1, 1 << 24, (n,), device="cuda", dtype=torch.int32).float() * 64.0
+    eb = 0.5
+    cap = pkg.max_stream_bytes(n)
+    chunks = lambda a, b, L: all(torch.equal(a[i:min(i + (1 << 28), L)], b[i:min(i + (1 << 28), L)])
+                                 for i in range(0, L, 1 << 28))
+    with pkg.Workspace(n) as ws:
+        s1 = torch.empty(cap, dtype=torch.uint8, device="cuda")
+        ws.compress(x, eb, s1)
+        L1 = ws.last_size()
+        assert L1 > (1 << 32) and L1 <= cap
+        dec = torch.empty(n, dtype=torch.float32, device="cuda")
+        ws.decompress(s1, L1, n, eb, dec)
+        torch.cuda.synchronize()
+        assert float((dec - x).abs().max()) <= 2 * eb      # within the bound (+ eb of float32 rounding, as the reference)
+        s2 = torch.empty(cap, dtype=torch.uint8, device="cuda")
+        ws.compress(dec, eb, s2)
+        assert ws.last_size() == L1 and chunks(s1, s2, L1)
+        # stream (+) floats and stream (+) stream meet in the same bytes
+        ws.hom_sum_f32(s1, L1, x, eb, s2)
+        L2 = ws.last_size()
+        s3 = torch.empty(cap, dtype=torch.uint8, device="cuda")
+        ws.hom_add(s1, L1, s1, L1, n, s3)
+        assert ws.last_size() == L2 and chunks(s2, s3, L2)
+        # and decode to twice the values (wrapping int32 is not reached: |2q| < 2^31)
+        out = torch.empty(n, dtype=torch.float32, device="cuda")
+        ws.decompress(s3, L2, n, eb, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, 2 * dec)
