@@ -224,6 +224,18 @@ def main() -> int:
     add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n)
     add("hom_add", lambda: ws.hom_add(cmp_a, la, cmp_b, lb, n, cmp_s), la + lb + ls)
     torch.cuda.synchronize()
+
+    # The workflow the homomorphic sum replaces, as the reference's evaluator times it
+    # (decompress, operate, compress: HomComp/src/homcomp_eval.cu:189-203, against
+    # homomorphic_sum_F :205-209, speedup printed at :225): same operands, same bound.
+    def doc_workflow():
+        ws.decompress(cmp_a, la, n, eb, dec)
+        dec.add_(y)
+        ws.compress(dec, eb, cmp_b)
+
+    ms_doc = time_op(torch, doc_workflow, max(3, it // 2))
+    ws.compress(y, eb, cmp_b)   # cmp_b holds compress(y) again
+    torch.cuda.synchronize()
     if args.copy_calibration:
         # a copy kernel of known size: reads 4N bytes and writes 4N bytes
         ms = time_op(torch, lambda: dec.copy_(x), 3)
@@ -250,6 +262,8 @@ def main() -> int:
         "compression_ratio_ref_convention": round(4 * n / pkg.ref_cmpsize(la, n), 3),
         "compression_ratio_sum": round(4 * n / ls, 3),
         "pct_hbm_peak": {k: round(100 * v["frac_hbm"], 2) for k, v in ops.items()},
+        "doc_workflow_ms": round(ms_doc, 4),
+        "hom_sum_speedup_over_doc_workflow": round(ms_doc / ops["hom_sum_f32"]["ms"], 2),
         "ops": ops,
         "roofline": roofline,
     }
