@@ -131,9 +131,11 @@ def error_measures(torch, x, y, dec, eb, chunk=1 << 24):
     cov = s_od / n - (s_o / n) * (s_d / n)
     var_o, var_d = s_oo / n - (s_o / n) ** 2, s_dd / n - (s_d / n) ** 2
     import math
-    # the reference quantises and dequantises in float32: each operand may exceed eb by 2^-21 of its
-    # magnitude, which the 0.1 % of slack covers for these inputs (the parity tests use the same)
-    return {"max_abs_err": dmax, "bound": 2 * eb, "within_bound": bool(dmax <= 2 * eb * (1 + 1e-3)),
+    # the reference quantises and dequantises in float32, so each operand's reconstruction carries
+    # two float32 roundings besides the bound: up to one unit in the last place of its magnitude,
+    # which shows once eb comes within a few hundred such units (REL 1e-6)
+    slack = max(abs(lo), abs(hi)) * 2.0 ** -23
+    return {"max_abs_err": dmax, "bound": 2 * eb, "float32_slack": slack, "within_bound": bool(dmax <= 2 * eb + slack),
             "psnr_db": round(20 * math.log10(rng) - 10 * math.log10(mse), 3) if mse > 0 and rng > 0 else None,
             "nrmse": math.sqrt(mse) / rng if rng > 0 else None,
             "correlation": round(cov / math.sqrt(var_o * var_d), 9) if var_o > 0 and var_d > 0 else None}

@@ -293,11 +293,11 @@ def test_many_rounds_and_small_grids(pkg, cuda, orc, gen, monkeypatch, grid_perc
         g.close()
 
 
-@pytest.mark.parametrize("stage,slots", [("small", 2), ("large", 2), ("small", 3), ("small", 4), ("large", 4)])
+@pytest.mark.parametrize("stage,slots", [("small", 2), ("medium", 2), ("large", 2), ("small", 3), ("medium", 3), ("small", 4), ("large", 4)])
 def test_lds_budgets_and_deferral_depths(pkg, cuda, orc, gen, monkeypatch, stage, slots):
     """Every LDS budget (HOMCOMP_STAGE) and deferral depth (HOMCOMP_SLOTS) gives the same bytes:
-    with the small budget and many slots most tiles of poorly compressible data outgrow their LDS
-    slot and travel through the spill area, with the large one they stay in LDS."""
+    with the small and medium budgets and many slots most tiles of poorly compressible data outgrow
+    their LDS slot and travel through the spill area, with the large one they stay in LDS."""
     monkeypatch.setenv("HOMCOMP_STAGE", stage)
     monkeypatch.setenv("HOMCOMP_SLOTS", str(slots))
     orc.set_threads(16)
@@ -322,7 +322,7 @@ def test_lds_budgets_and_deferral_depths(pkg, cuda, orc, gen, monkeypatch, stage
 
 def test_lds_budget_follows_the_data(pkg, cuda, orc, gen):
     """Without a forced budget a workspace starts compress with the large LDS budget and moves to
-    the small one once a finished call has shown the data to be compressible; alternating data
+    a smaller one once a finished call has shown the data to be compressible; alternating data
     families on one workspace must keep producing the oracle's bytes."""
     orc.set_threads(16)
     n = 1 << 21

@@ -52,12 +52,12 @@ struct homcomp_workspace {
     float *d_partial;         // min/max partials
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
-    uint32_t max_grid[hc::kOpCount][2];  // resident workgroups of each operation's kernel, per LDS budget (small, large)
+    uint32_t max_grid[hc::kOpCount][3];  // resident workgroups of each operation's kernel, per LDS budget (small, medium, large)
     uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint8_t *d_spill;         // spill slots: four worst-case tiles per data wave
     uint32_t out_slots;       // deferral depth of packed tiles (2..4)
-    int stage_class;          // -1: chosen per call; 0 / 1: HOMCOMP_STAGE=small / large forces one LDS budget
+    int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
 };
 
 namespace {
@@ -109,14 +109,19 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
                : HOMCOMP_ERR_HIP;
 }
 
-// LDS stage per data wave (two deferred tiles by default).  The small budgets fit tiles of streams
-// compressed about 4x or better and let more waves share a compute unit; the large one holds
-// tiles down to a ratio of 2 (2.1 with two incoming streams, whose kernel holds more LDS of its
-// own: with the full 8 KiB slots only one of its workgroups fits a compute unit, and that is
-// slower than spilling).  A tile beyond its slot still works (it goes through the spill area),
-// only slower, so the choice below is a performance heuristic, never a correctness matter.
-constexpr uint32_t kStageSmall[hc::kOpCount] = {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)};
-constexpr uint32_t kStageLarge[hc::kOpCount] = {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7680 + 64)};
+// LDS stage per data wave (two deferred tiles by default), in three budgets that let 4, 3 and 2
+// workgroups share a compute unit (with the LDS the kernels hold besides: 0.6 KiB for compress,
+// 12.5 KiB with one incoming stream, 15.8 KiB with two).  The slots hold tiles of streams
+// compressed about 4.6x / 2.9x / 2x or better for compress, 6x / 3.7x / 2x for the sums with one
+// incoming stream and 9x / 4x / 2.1x with two.  A tile beyond its slot still works (it goes
+// through the spill area), only slower, so the choice below is a performance heuristic, never a
+// correctness matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
+// fits a compute unit, which is slower than spilling: its largest slots are 7.5 KiB.)
+constexpr int kStageClasses = 3;
+constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
+    {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
+    {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4544 + 64)},
+    {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7680 + 64)}};
 
 // The stream-producing kernels of this process never overlap on a device.  Each of them needs
 // its whole grid resident (the scan's waits), and two such grids from different streams can each
@@ -165,17 +170,20 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
 {
     p.spill = ws->d_spill;
     p.out_slots = ws->out_slots;
-    int cls = 1;
+    int cls = kStageClasses - 1;
     if (op == hc::kOpDecompress) {
         cls = 0;
     } else {
         if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
-        const uint64_t slot_cap = kStageSmall[op] / ws->out_slots - 64u;
-        if (expected_tile_bytes != 0 && expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) cls = 0;
+        // the smallest budget whose slots hold the expected tile with an eighth to spare
+        for (int c = kStageClasses - 2; c >= 0 && expected_tile_bytes != 0; --c) {
+            const uint64_t slot_cap = kStage[c][op] / ws->out_slots - 64u;
+            if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) cls = c;
+        }
         if (ws->stage_class >= 0) cls = ws->stage_class;
         p.host_total = &ws->h_mean_tile[op];
     }
-    p.stage_bytes = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge[op] : kStageSmall[op]);
+    p.stage_bytes = op == hc::kOpDecompress ? 0u : kStage[cls][op];
     if (op == hc::kOpDecompress) return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     return chained_launch(ws, op, p, ws->max_grid[op][cls], s);
 }
@@ -266,9 +274,9 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     bool ok = hip_ok(hipGetDeviceProperties(&prop, ws->device));
     uint32_t widest = 0;
     for (int op = 0; ok && op < hc::kOpCount; ++op) {
-        for (int cls = 0; ok && cls < 2; ++cls) {
+        for (int cls = 0; ok && cls < kStageClasses; ++cls) {
             int per_cu = 0;
-            const uint32_t stage = op == hc::kOpDecompress ? 0u : (cls ? kStageLarge[op] : kStageSmall[op]);
+            const uint32_t stage = op == hc::kOpDecompress ? 0u : kStage[cls][op];
             ok = hip_ok(hc::op_kernel_residency(op, stage, &per_cu));
             if (ok && per_cu < 1) per_cu = 1;
             // one compute unit's worth of workgroups is left free: the persistent grid must be fully
@@ -295,7 +303,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     ws->stage_class = -1;
     if (const char *e = std::getenv("HOMCOMP_STAGE")) {
         if (std::strcmp(e, "small") == 0) ws->stage_class = 0;
-        if (std::strcmp(e, "large") == 0) ws->stage_class = 1;
+        if (std::strcmp(e, "medium") == 0) ws->stage_class = 1;
+        if (std::strcmp(e, "large") == 0) ws->stage_class = 2;
     }
     ws->out_slots = 2;
     if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
