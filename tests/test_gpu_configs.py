@@ -199,12 +199,18 @@ def test_stream_longer_than_4_gib(pkg, cuda):
     """Maximum sizes: 2^30 + 12345 incompressible values give a stream of 4.3e9 bytes, beyond the
     32-bit offsets of the reference (HomComp/src/GSZ.cu:170-239 keeps them in unsigned int); the
     offsets here are 64-bit.  No CPU pass at this size: the checks are properties of the codec.
-    Values are multiples of 64 below 2^30 with eb = 0.5: the quantised values survive the trip
-    through float32 (the reference's two float roundings move negative values by one, which float32
-    holds or rounds back), so compress(decompress(s)) must give s back byte for byte."""
+    Values are +-64 m with 2^18 <= m < 2^24 and eb = 0.5: the quantised values survive the trip
+    through float32 (the reference's two float roundings move negative values of 2^24 and more by
+    one, which float32 rounds back), so compress(decompress(s)) must give s back byte for byte.
+    Magnitudes below 2^24 are left out because they are not moved: a delta between one of them and
+    a value 2^30 away would be 2^30 exactly, and twice that is the one int32 the 5-bit plane count
+    cannot hold (HomComp/src/GSZ.cu:163)."""
     torch = cuda
     n = (1 << 30) + 12345
-    x = torch.randint(-(1 << 24) + 1, 1 << 24, (n,), device="cuda", dtype=torch.int32).float() * 64.0
+    torch.manual_seed(20)
+    x = torch.randint(1 << 18, 1 << 24, (n,), device="cuda", dtype=torch.int32)
+    x *= torch.randint(0, 2, (n,), device="cuda", dtype=torch.int32) * 2 - 1
+    x = x.float() * 64.0
     eb = 0.5
     cap = pkg.max_stream_bytes(n)
     chunks = lambda a, b, L: all(torch.equal(a[i:min(i + (1 << 28), L)], b[i:min(i + (1 << 28), L)])

@@ -290,30 +290,47 @@ __device__ __forceinline__ void unpack_group(const uint8_t *stage, uint32_t base
     }
 }
 
-// Decodes the lane's eight deltas of a block and adds them to v[] (wrapping).
-__device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0, uint32_t hdr,
-                                            bool active, int k, int32_t v[8])
+// What the decoder needs of a header byte, in one byte: bits 0-4 the plane count F, bits 5-7 the
+// number of outlier bytes (0 in plain mode, 1-4 in outlier mode).  0 for a block without payload.
+__device__ __forceinline__ uint32_t header_digest(uint32_t h)
 {
-    if (!active) hdr = 0;
-    const uint32_t sel = hdr >> 7;
-    const uint32_t F = hdr & 0x1fu;
-    const uint32_t ob = sel ? ((hdr >> 5) & 3u) + 1u : 0u;
+    const uint32_t F = h & 0x1fu;
+    const uint32_t ob = (h & 0x80u) ? ((h >> 5) & 3u) + 1u : 0u;
+    return F | (ob << 5);
+}
+
+// (a ^ b) + c in one instruction
+__device__ __forceinline__ uint32_t xor_add(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t r;
+    asm("v_xad_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Decodes the lane's eight deltas of a block and adds them to v[] (wrapping).  `digest` is
+// header_digest() of the block's header byte, or 0 for a block that is not to be read.
+__device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0, uint32_t digest, int k, int32_t v[8])
+{
+    const uint32_t F = digest & 0x1fu;
+    const uint32_t ob = digest >> 5;
     const uint32_t base = pos0 + ob + 4u + (uint32_t)k;
     uint32_t a[8];
     unpack_group<0>(stage, base, F < 8u ? F : 8u, a);
     if (F > 8u) unpack_group<1>(stage, base, F < 16u ? F - 8u : 8u, a);
     if (F > 16u) unpack_group<2>(stage, base, F < 24u ? F - 16u : 8u, a);
     if (F > 24u) unpack_group<3>(stage, base, F - 24u, a);
-    const uint32_t sb = hdr ? stage[pos0 + ob + (uint32_t)k] : 0u;   // :921-924, :990-994
+    const uint32_t sb = digest ? stage[pos0 + ob + (uint32_t)k] : 0u;   // :921-924, :990-994
     // outlier: lane k reads byte k, the quad ORs the pieces together (:913-917, :986-987, :1005-1006)
     const uint32_t piece = (uint32_t)k < ob ? (uint32_t)stage[pos0 + (uint32_t)k] << (8 * k) : 0u;
     const uint32_t o = quad_or(piece);
-    if (sel && k == 0) a[0] = o;
+    if (ob != 0u && k == 0) a[0] = o;
 #pragma unroll
     for (int m = 0; m < 8; ++m) {                         // :1432-1434
-        const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)sb, 7 - m, 1);   // 0 or ~0
-        // v + ((a ^ mask) - mask), in the order that is one xor-add
-        v[m] = (int32_t)((a[m] ^ mask) + ((uint32_t)v[m] - mask));
+        uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)sb, 7 - m, 1);   // 0 or ~0
+        // v + ((a ^ mask) - mask): a subtraction and one xor-add.  (Where the compiler sees where
+        // the mask comes from it extracts the bit a second time to add it instead.)
+        asm("" : "+v"(mask));
+        v[m] = (int32_t)xor_add(a[m], mask, (uint32_t)v[m] - mask);
     }
 }
 

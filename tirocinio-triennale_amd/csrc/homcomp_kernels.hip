@@ -382,11 +382,16 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     const uint32_t incl = wave_incl_scan_u32(z0 + z1, lane);
                     const uint32_t o0 = incl - z0 - z1, o1 = o0 + z0;
                     *reinterpret_cast<uint32_t *>(&s_ofs_in[wave][c][b][2 * lane]) = o0 | (o1 << 16);
-                    *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)hdr_next[c];
                     if ((lane & 7) == 0) s_rel[wave][c][b][lane >> 3] = o0;
                     if (lane == 63) s_rel[wave][c][b][kSub] = incl;
                     const uint64_t room64 = p.in_size[c] > start_next[c] ? p.in_size[c] - start_next[c] : 0u;
                     const uint32_t room = room64 > 0xffff0000ull ? 0xffff0000u : (uint32_t)room64;
+                    // what the sub-steps need of the header bytes; a block without payload, or one
+                    // that starts at or beyond the stated size (out-of-bound rule of
+                    // HomComp/src/GSZ.cu:908-911 on the absolute payload offset), is not read
+                    const uint32_t d0 = z0 != 0u && o0 < room ? header_digest(h0) : 0u;
+                    const uint32_t d1 = z1 != 0u && o1 < room ? header_digest(h1) : 0u;
+                    *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
                     if (b) {
                         start_ctx1[c] = start_next[c];
                         room_ctx1[c] = room;
@@ -559,11 +564,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         request_in(c, r2, b2, s2, in);
                         wave_lds_fence();
                         // ---- decode (HomComp/src/GSZ.cu:883-1434)
-                        const uint32_t h = s_hdr_in[wave][c][buf][blk];
+                        const uint32_t digest = s_hdr_in[wave][c][buf][blk];
                         const uint32_t ofs = s_ofs_in[wave][c][buf][blk];
-                        // out-of-bound rule of HomComp/src/GSZ.cu:908-911 on the absolute payload offset
-                        const bool active = size_from_header(h) != 0u && ofs < (buf ? room_ctx1[c] : room_ctx0[c]);
-                        unpack8_add(st, shift + ofs - rel0, h, active, k, v);
+                        unpack8_add(st, shift + ofs - rel0, digest, k, v);
                         wave_lds_fence();   // the stage is rewritten by the next stream and the next sub-step
                     }
                 }
