@@ -520,6 +520,16 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             const uint64_t tile_elem0 = (uint64_t)t0 * kTileElems;
             // sub-step s of this tile; (r2, b2, s2) is the sub-step the freed registers are requested for
             auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2) __attribute__((always_inline)) {
+                // the blocks' digests and offsets first: nothing in the sub-step writes them, and
+                // read here they are on their way while the wave waits for its operands
+                uint32_t digest[kIn], ofs[kIn];
+                if constexpr (NIN > 0) {
+#pragma unroll
+                    for (int c = 0; c < NIN; ++c) {
+                        digest[c] = s_hdr_in[wave][c][buf][s * 16 + quad];
+                        ofs[c] = s_ofs_in[wave][c][buf][s * 16 + quad];
+                    }
+                }
                 // elements beyond the end arrive as zeros (0.0f quantises to 0), as the reference pads
                 int32_t v[8];
                 if constexpr (LOCAL == kLocalF32) {
@@ -544,7 +554,6 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                 }
                 request_local(r2, s2, loc);
                 if constexpr (NIN > 0) {
-                    const int blk = s * 16 + quad;
 #pragma unroll
                     for (int c = 0; c < NIN; ++c) {
                         // ---- the sub-step's payload range: registers -> LDS stage
@@ -564,9 +573,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         request_in(c, r2, b2, s2, in);
                         wave_lds_fence();
                         // ---- decode (HomComp/src/GSZ.cu:883-1434)
-                        const uint32_t digest = s_hdr_in[wave][c][buf][blk];
-                        const uint32_t ofs = s_ofs_in[wave][c][buf][blk];
-                        unpack8_add(st, shift + ofs - rel0, digest, k, v);
+                        unpack8_add(st, shift + ofs[c] - rel0, digest[c], k, v);
                         wave_lds_fence();   // the stage is rewritten by the next stream and the next sub-step
                     }
                 }
