@@ -235,6 +235,25 @@ def test_unaligned_stream_pointers(gpu, orc, gen, offset):
     assert_stream_equal(gpu.hom_sum_f32(want, y, eb, offset=offset), orc.hom_sum_f32(want, y, eb), "hom")
 
 
+@pytest.mark.parametrize("tiles,offset", [(2047, 0), (2048, 0), (2048, 3), (2049, 0), (2049, 5)])
+def test_offsets_prepass_sizes(pkg, cuda, orc, gen, tiles, offset):
+    """The offsets of an incoming stream's tiles are computed ahead of the tile kernel in blocks of
+    256 tiles: eight blocks and a ninth with one tile, aligned and unaligned stream pointers,
+    ragged last tile."""
+    orc.set_threads(16)
+    n = tiles * 4096 - 37
+    x, y = gen.smooth_np(n, 70), gen.gradient_like_np(n, 71)
+    eb = np.float32(3e-4)
+    g = Gpu(pkg, cuda, n)
+    try:
+        sx = orc.compress(x, eb)
+        assert_stream_equal(g.hom_sum_f32(sx, y, eb, offset=offset), orc.hom_sum_f32(sx, y, eb), "hom_sum_f32")
+        dec = g.decompress(sx, n, eb, offset=offset)
+        assert np.array_equal(dec.view(np.uint32), orc.decompress(sx, n, eb).view(np.uint32))
+    finally:
+        g.close()
+
+
 def test_value_range(gpu, orc, gen, pkg):
     for kind, n in (("smooth", 1 << 20), ("uniform", 12345), ("gradient_like", 7)):
         x = make(gen, kind, n, seed=4)
