@@ -174,6 +174,20 @@ __device__ __forceinline__ void transpose8(uint32_t &lo, uint32_t &hi)
     hi ^= t >> 4;
 }
 
+// The same for blocks of at most four planes, in one register: eight 4-bit values as
+// [4 bytes][2 nibbles][4 bits], byte r = value 7-r in the low and value 3-r in the high nibble.
+// Swapping the byte index with the bit index inside the nibble (two delta swaps) leaves plane p in
+// byte p with the bit of value m at position 7-m; the same two swaps lead back.
+__device__ __forceinline__ uint32_t transpose4(uint32_t y)
+{
+    uint32_t t;
+    t = (y ^ (y >> 7)) & 0x00AA00AAu;
+    y ^= t ^ (t << 7);
+    t = (y ^ (y >> 14)) & 0x0000CCCCu;
+    y ^= t ^ (t << 14);
+    return y;
+}
+
 // ---------------------------------------------------------------- per-lane block pieces
 
 // Encoder front end for one lane's 8 signed deltas (HomComp/src/GSZ.cu:86-164): sign byte,
@@ -245,10 +259,27 @@ __device__ __forceinline__ void pack_group(Bytes stage, uint32_t base, const uin
         stage[base + 4u * (uint32_t)(8 * G + r)] = (uint8_t)((r < 4 ? lo : hi) >> (8 * (r & 3)));
 }
 
+// Planes 0-3 of a block whose values are all below 16.
+template <typename Bytes>
+__device__ __forceinline__ void pack_low4(Bytes stage, uint32_t base, const uint32_t a[8])
+{
+    constexpr uint32_t two = 0x0c0c0400u;
+    const uint32_t lo = __builtin_amdgcn_perm(__builtin_amdgcn_perm(a[4], a[5], two),
+                                              __builtin_amdgcn_perm(a[6], a[7], two), 0x05040100u);
+    const uint32_t hi = __builtin_amdgcn_perm(__builtin_amdgcn_perm(a[0], a[1], two),
+                                              __builtin_amdgcn_perm(a[2], a[3], two), 0x05040100u);
+    const uint32_t y = transpose4(lo | (hi << 4));
+#pragma unroll
+    for (int r = 3; r >= 0; --r) stage[base + 4u * (uint32_t)r] = (uint8_t)(y >> (8 * r));
+}
+
 template <typename Bytes>
 __device__ __forceinline__ void pack8(Bytes stage, uint32_t pos0, uint32_t hdr, int k,
                                       const uint32_t a_in[8], uint32_t sb, uint32_t a0)
 {
+    // no block of the wave has more than four planes (the usual case at moderate error bounds):
+    // half the stores and a third of the transposition
+    const bool low = __builtin_amdgcn_ballot_w64((hdr & 0x1fu) > 4u) == 0;
     if (hdr == 0) return;                                 // zero block (:287)
     const uint32_t sel = hdr >> 7;
     const uint32_t F = hdr & 0x1fu;
@@ -258,10 +289,14 @@ __device__ __forceinline__ void pack8(Bytes stage, uint32_t pos0, uint32_t hdr, 
     for (int m = 1; m < 8; ++m) a[m] = a_in[m];
     a[0] = (sel && k == 0) ? 0u : a_in[0];                // element 0 leaves the planes (:274)
     const uint32_t base = pos0 + ob + 4u + (uint32_t)k;
-    if (F > 24u) pack_group<3>(stage, base, a);
-    if (F > 16u) pack_group<2>(stage, base, a);
-    if (F > 8u) pack_group<1>(stage, base, a);
-    pack_group<0>(stage, base, a);
+    if (low) {
+        pack_low4(stage, base, a);
+    } else {
+        if (F > 24u) pack_group<3>(stage, base, a);
+        if (F > 16u) pack_group<2>(stage, base, a);
+        if (F > 8u) pack_group<1>(stage, base, a);
+        pack_group<0>(stage, base, a);
+    }
     stage[pos0 + ob + (uint32_t)k] = (uint8_t)sb;         // sign word, MSB = element 0 (:292-295)
     if ((uint32_t)k < ob) stage[pos0 + (uint32_t)k] = (uint8_t)(a0 >> (8 * k));   // little-endian outlier (:271-275)
 }
@@ -290,6 +325,20 @@ __device__ __forceinline__ void unpack_group(const uint8_t *stage, uint32_t base
     }
 }
 
+// Planes 0-3 only, for a wave in which no block has more: four bytes, one register.
+__device__ __forceinline__ void unpack_low4(const uint8_t *stage, uint32_t base, uint32_t width, uint32_t a[8])
+{
+    uint32_t y = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) y |= (uint32_t)stage[base + 4u * (uint32_t)r] << (8 * r);
+    y = transpose4(y);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        a[7 - r] = __builtin_amdgcn_ubfe(y, 8 * r, width);
+        a[3 - r] = __builtin_amdgcn_ubfe(y, 8 * r + 4, width);
+    }
+}
+
 // What the decoder needs of a header byte, in one byte: bits 0-4 the plane count F, bits 5-7 the
 // number of outlier bytes (0 in plain mode, 1-4 in outlier mode).  0 for a block without payload.
 __device__ __forceinline__ uint32_t header_digest(uint32_t h)
@@ -311,14 +360,20 @@ __device__ __forceinline__ uint32_t xor_add(uint32_t a, uint32_t b, uint32_t c)
 // header_digest() of the block's header byte, or 0 for a block that is not to be read.
 __device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0, uint32_t digest, int k, int32_t v[8])
 {
+    // sixteen blocks without payload (long runs of them make up streams of sparse data): nothing to add
+    if (__builtin_amdgcn_ballot_w64(digest != 0u) == 0) return;
     const uint32_t F = digest & 0x1fu;
     const uint32_t ob = digest >> 5;
     const uint32_t base = pos0 + ob + 4u + (uint32_t)k;
     uint32_t a[8];
-    unpack_group<0>(stage, base, F < 8u ? F : 8u, a);
-    if (F > 8u) unpack_group<1>(stage, base, F < 16u ? F - 8u : 8u, a);
-    if (F > 16u) unpack_group<2>(stage, base, F < 24u ? F - 16u : 8u, a);
-    if (F > 24u) unpack_group<3>(stage, base, F - 24u, a);
+    if (__builtin_amdgcn_ballot_w64(F > 4u) == 0) {   // wave-uniform
+        unpack_low4(stage, base, F, a);
+    } else {
+        unpack_group<0>(stage, base, F < 8u ? F : 8u, a);
+        if (F > 8u) unpack_group<1>(stage, base, F < 16u ? F - 8u : 8u, a);
+        if (F > 16u) unpack_group<2>(stage, base, F < 24u ? F - 16u : 8u, a);
+        if (F > 24u) unpack_group<3>(stage, base, F - 24u, a);
+    }
     const uint32_t sb = digest ? stage[pos0 + ob + (uint32_t)k] : 0u;   // :921-924, :990-994
     // outlier: lane k reads byte k, the quad ORs the pieces together (:913-917, :986-987, :1005-1006)
     const uint32_t piece = (uint32_t)k < ob ? (uint32_t)stage[pos0 + (uint32_t)k] << (8 * k) : 0u;
