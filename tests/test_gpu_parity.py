@@ -109,11 +109,12 @@ def test_hom_sums(gpu, orc, gen, kind, n, mode, val):
     assert (np.abs(dec.astype(np.float64) - s) <= bound).all()
 
 
-def rand_deltas(rng, nblocks):
-    """Blocks covering every plane count, both modes and every outlier width."""
+def rand_deltas(rng, nblocks, caps=None):
+    """Blocks covering every plane count, both modes and every outlier width.  With caps, the
+    plane counts of blocks 16 g .. 16 g + 15 (one step of a wave) stay at or below caps[g]."""
     d = np.zeros((nblocks, 32), np.int64)
     for b in range(nblocks):
-        F = int(rng.integers(0, 32))
+        F = int(rng.integers(0, 32)) if caps is None else int(rng.integers(0, caps[b // 16] + 1))
         mode = int(rng.integers(0, 5))
         if F:
             d[b] = rng.integers(0, 1 << F, 32)
@@ -153,6 +154,28 @@ def test_every_rate_and_mode(gpu, orc):
     # and decompress of the crafted stream (quantised values = running sums)
     dec = gpu.decompress(s1, n, 0.5)
     assert np.array_equal(dec.view(np.uint32), orc.decompress(s1, n, 0.5).view(np.uint32))
+
+
+def test_few_planes_per_step(gpu, orc):
+    """Steps of sixteen blocks whose plane counts all stay at or below 0, 1, .. 6, 8 or 9: steps
+    with at most four planes take the one-register pack and unpack, steps of empty blocks skip
+    the decoder, and both sit next to steps of the general kind in the same tile.  Outlier
+    mode (a large first element with few planes behind it) is part of every kind."""
+    rng = np.random.default_rng(17)
+    n = 1 << 17
+    groups = n // 512
+    for trial in range(3):
+        caps = rng.choice([0, 1, 2, 3, 4, 4, 4, 5, 6, 8, 9], groups)
+        caps2 = rng.choice([0, 0, 1, 2, 3, 4, 4, 5, 9], groups)
+        d1 = rand_deltas(rng, n // 32, caps) >> 1
+        d2 = rand_deltas(rng, n // 32, caps2) >> 1
+        zero = orc.compress(np.zeros(n, np.float32), 1.0)
+        s1, s2 = orc.encode_deltas(d1), orc.encode_deltas(d2)
+        assert_stream_equal(gpu.hom_sum_i32(zero, d1), s1, f"encode #{trial}")
+        assert_stream_equal(gpu.hom_sum_i32(s2, d1), orc.encode_deltas(d1 + d2), f"hom_sum_i32 #{trial}")
+        assert_stream_equal(gpu.hom_add(s1, s2, n), orc.encode_deltas(d1 + d2), f"hom_add #{trial}")
+        dec = gpu.decompress(s1, n, 0.5)
+        assert np.array_equal(dec.view(np.uint32), orc.decompress(s1, n, 0.5).view(np.uint32)), f"decompress #{trial}"
 
 
 def test_zero_incoming_blocks(gpu, orc, gen):
