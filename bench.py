@@ -225,6 +225,13 @@ def main() -> int:
     add("hom_sum_f32", lambda: ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s), la + 4 * n + ls)
     add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n)
     add("hom_add", lambda: ws.hom_add(cmp_a, la, cmp_b, lb, n, cmp_s), la + lb + ls)
+    # the integer-delta variant of the sum with its Lorenzo pre-pass, and the min/max scan behind REL bounds
+    dlt = torch.empty(n, dtype=torch.int32, device="cuda")
+    add("quant_predict", lambda: pkg.quant_predict(y, eb, dlt), 8 * n)
+    add("hom_sum_i32", lambda: ws.hom_sum_i32(cmp_a, la, dlt, cmp_b), la + 4 * n + ls)
+    add("value_range", lambda: ws.value_range(x, mm[0:2]), 4 * n)
+    del dlt
+    ws.compress(y, eb, cmp_b)   # cmp_b holds compress(y) again
     torch.cuda.synchronize()
 
     # The workflow the homomorphic sum replaces, as the reference's evaluator times it
