@@ -307,31 +307,29 @@ __device__ __forceinline__ void pack8(Bytes stage, uint32_t pos0, uint32_t hdr, 
 // first eight plane bytes are always read (up to 35 bytes past the block's end, inside the
 // stage's slack) and the planes the block does not have are cut off when the bits are extracted.
 // Must run with all lanes of the wave active (the outlier bytes are gathered across the quad).
-template <int G>
-__device__ __forceinline__ void unpack_group(const uint8_t *stage, uint32_t base, uint32_t width, uint32_t a[8])
+// Four bytes, each in a register of its own, as one word (byte 0 first): three byte permutes.
+__device__ __forceinline__ uint32_t word_of_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3)
 {
-    uint32_t lo = 0, hi = 0;
+    return __builtin_amdgcn_perm(__builtin_amdgcn_perm(b3, b2, 0x0c0c0400u), __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u),
+                                 0x05040100u);
+}
+
+// Planes 8G..8G+7 of the lane's eight values: byte r of (lo, hi) = those planes of value 7-r.
+template <int G>
+__device__ __forceinline__ void load_group(const uint8_t *stage, uint32_t base, uint32_t &lo, uint32_t &hi)
+{
+    uint32_t b[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        const uint32_t byte = stage[base + 4u * (uint32_t)(8 * G + r)];
-        if (r < 4) lo |= byte << (8 * r); else hi |= byte << (8 * (r - 4));
-    }
+    for (int r = 0; r < 8; ++r) b[r] = stage[base + 4u * (uint32_t)(8 * G + r)];
+    lo = word_of_bytes(b[0], b[1], b[2], b[3]);
+    hi = word_of_bytes(b[4], b[5], b[6], b[7]);
     transpose8(lo, hi);
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        // byte r = the block's planes 8G..8G+7 of element 7-r; only `width` of them exist
-        const uint32_t bits = __builtin_amdgcn_ubfe(r < 4 ? lo : hi, 8 * (r & 3), width);
-        a[7 - r] = G == 0 ? bits : a[7 - r] | (bits << (8 * G));
-    }
 }
 
 // Planes 0-3 only, for a wave in which no block has more: four bytes, one register.
 __device__ __forceinline__ void unpack_low4(const uint8_t *stage, uint32_t base, uint32_t width, uint32_t a[8])
 {
-    uint32_t y = 0;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) y |= (uint32_t)stage[base + 4u * (uint32_t)r] << (8 * r);
-    y = transpose4(y);
+    const uint32_t y = transpose4(word_of_bytes(stage[base], stage[base + 4u], stage[base + 8u], stage[base + 12u]));
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         a[7 - r] = __builtin_amdgcn_ubfe(y, 8 * r, width);
@@ -369,10 +367,43 @@ __device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0,
     if (__builtin_amdgcn_ballot_w64(F > 4u) == 0) {   // wave-uniform
         unpack_low4(stage, base, F, a);
     } else {
-        unpack_group<0>(stage, base, F < 8u ? F : 8u, a);
-        if (F > 8u) unpack_group<1>(stage, base, F < 16u ? F - 8u : 8u, a);
-        if (F > 16u) unpack_group<2>(stage, base, F < 24u ? F - 16u : 8u, a);
-        if (F > 24u) unpack_group<3>(stage, base, F - 24u, a);
+        // Groups of eight planes: a lane reads the groups its block has; the bytes of a value are
+        // then put together for as many groups as the widest block of the wave has, and the
+        // planes a block does not have (stray bytes, or the zeros of a group not read) are cut off
+        // in one extract of F bits.
+        uint32_t lo[4] = {0u, 0u, 0u, 0u}, hi[4] = {0u, 0u, 0u, 0u};
+        load_group<0>(stage, base, lo[0], hi[0]);
+        if (F > 8u) load_group<1>(stage, base, lo[1], hi[1]);
+        if (F > 16u) load_group<2>(stage, base, lo[2], hi[2]);
+        if (F > 24u) load_group<3>(stage, base, lo[3], hi[3]);
+        const bool any8 = __builtin_amdgcn_ballot_w64(F > 8u) != 0;
+        const bool any16 = __builtin_amdgcn_ballot_w64(F > 16u) != 0;
+        const bool any24 = __builtin_amdgcn_ballot_w64(F > 24u) != 0;
+        // byte j of the second, then of the first operand
+        auto two = [](int j) { return 0x0c0c0400u + 0x0101u * (uint32_t)j; };
+        auto sel = [](const uint32_t (&w)[4], const uint32_t (&v)[4], int g, int r) { return r < 4 ? w[g] : v[g]; };
+        if (!any8) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) a[7 - r] = __builtin_amdgcn_ubfe(sel(lo, hi, 0, r), 8 * (r & 3), F);
+        } else if (any24) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t x01 = __builtin_amdgcn_perm(sel(lo, hi, 1, r), sel(lo, hi, 0, r), two(r & 3));
+                const uint32_t x23 = __builtin_amdgcn_perm(sel(lo, hi, 3, r), sel(lo, hi, 2, r), two(r & 3));
+                a[7 - r] = __builtin_amdgcn_ubfe(__builtin_amdgcn_perm(x23, x01, 0x05040100u), 0, F);
+            }
+        } else if (any16) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t x01 = __builtin_amdgcn_perm(sel(lo, hi, 1, r), sel(lo, hi, 0, r), two(r & 3));
+                const uint32_t x = __builtin_amdgcn_perm(sel(lo, hi, 2, r), x01, 0x0c000100u + ((uint32_t)(4 + (r & 3)) << 16));
+                a[7 - r] = __builtin_amdgcn_ubfe(x, 0, F);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                a[7 - r] = __builtin_amdgcn_ubfe(__builtin_amdgcn_perm(sel(lo, hi, 1, r), sel(lo, hi, 0, r), two(r & 3)), 0, F);
+        }
     }
     const uint32_t sb = digest ? stage[pos0 + ob + (uint32_t)k] : 0u;   // :921-924, :990-994
     // outlier: lane k reads byte k, the quad ORs the pieces together (:913-917, :986-987, :1005-1006)
