@@ -27,7 +27,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X published peak
 # HBM bytes per launch of the dominant kernel (hom_sum_f32) measured with rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE and scaled as described in profiles/pmc_hbm_traffic_smooth_1GiB_rel1e-4.txt;
 # keyed by (kind, log2n, rel).  Other workloads report null.
-MEASURED_TRAFFIC = {("smooth", 28, 1e-4): 1.3436e+09}
+MEASURED_TRAFFIC = {("smooth", 28, 1e-4): 1.3437e+09}
 
 
 def time_op(torch, fn, iters: int) -> float:
