@@ -114,8 +114,8 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 // 12.5 KiB with one incoming stream, 15.8 KiB with two).  The slots hold tiles of streams
 // compressed about 4.6x / 2.9x / 2x or better for compress, 6x / 3.7x / 2x for the sums with one
 // incoming stream and 9x / 4x / 2.1x with two.  A tile beyond its slot still works (it goes
-// through the spill area), only slower, so the choice below is a performance heuristic, never a
-// correctness matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
+// through the spill area), so the choice below is a performance heuristic, never a correctness
+// matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
 // fits a compute unit, which is slower than spilling: its largest slots are 7.5 KiB.)
 constexpr int kStageClasses = 3;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
@@ -175,10 +175,20 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         cls = 0;
     } else {
         if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
-        // the smallest budget whose slots hold the expected tile with an eighth to spare
-        for (int c = kStageClasses - 2; c >= 0 && expected_tile_bytes != 0; --c) {
-            const uint64_t slot_cap = kStage[c][op] / ws->out_slots - 64u;
-            if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) cls = c;
+        if (expected_tile_bytes != 0) {
+            // the smallest budget whose slots hold the expected tile with an eighth to spare
+            int holds = -1;
+            for (int c = kStageClasses - 1; c >= 0; --c) {
+                const uint64_t slot_cap = kStage[c][op] / ws->out_slots - 64u;
+                if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) holds = c;
+            }
+            // Tiles that no budget holds go through the spill area whatever the choice: the most
+            // waves, then.  The sums are bound by instruction issue and gain more from a third and
+            // fourth workgroup per compute unit than they lose by spilling, so they never take the
+            // large budget by themselves; compress is bound by memory and avoids the spill traffic
+            // where it can.  (Measured on MI355X at 1 GiB, compression ratios 1.6 to 4.4.)
+            cls = holds < 0 ? 0 : holds;
+            if (cls == kStageClasses - 1 && op != hc::kOpCompress) cls = 0;
         }
         if (ws->stage_class >= 0) cls = ws->stage_class;
         p.host_total = &ws->h_mean_tile[op];

@@ -277,30 +277,52 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_wave_barrier();
 }
 
-// Copy of a spilled tile from the wave's slot of the spill area to its place in the stream.  The
-// slot is read with device-scope loads (it was written by this wave, but an older copy of the
-// line may sit in the vector cache from the slot's previous use).
+// Whole 16-byte pieces from the front of a wave's LDS slot to its spill slot (both 16-byte aligned).
+__device__ __forceinline__ void spill_pieces(const uint8_t *stage, uint8_t *slot_at, uint32_t bytes, int lane)
+{
+    for (uint32_t i = 16u * (uint32_t)lane; i < bytes; i += 1024u)
+        *reinterpret_cast<u32x4 *>(slot_at + i) = *reinterpret_cast<const u32x4 *>(stage + i);
+}
+
+// Copy of a spilled tile from the wave's slot of the spill area to its place in the stream: like
+// copy_out, bytes up to the first 16-byte boundary of the destination, aligned 16-byte stores put
+// together from two aligned 16-byte pieces of the slot, then the remaining bytes.  The slot is
+// read with device-scope loads (it was written by this wave, but an older copy of a line may sit
+// in the vector cache from the slot's previous use).
 __device__ __forceinline__ void copy_out_spill(const uint8_t *slot, uint8_t *g, uint32_t tot, int lane)
 {
-    const uint32_t mis = (uint32_t)((uintptr_t)g & 3u);
-    uint32_t head = (4u - mis) & 3u;
+    const uint32_t mis = (uint32_t)((uintptr_t)g & 15u);
+    uint32_t head = (16u - mis) & 15u;
     if (head > tot) head = tot;
+    const uint32_t body = tot - head;
+    const uint32_t nch = body >> 4;
+    const uint32_t tail = body & 15u;
     const uint32_t *sw = reinterpret_cast<const uint32_t *>(slot);
-    auto word = [&](uint32_t w) { return __hip_atomic_load(sw + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    if ((uint32_t)lane < head) g[lane] = (uint8_t)(word(0) >> (8 * lane));
-    const uint32_t nw = (tot - head) >> 2;
-    const uint32_t tail = (tot - head) & 3u;
-    const uint32_t sh = head & 3u;
-    for (uint32_t c = lane; c < nw; c += 64) {
-        const uint32_t s = head + 4u * c;
-        const uint32_t w0 = s >> 2;
-        const uint32_t x0 = word(w0), x1 = word(w0 + 1);
-        *reinterpret_cast<uint32_t *>(g + s) = __builtin_amdgcn_alignbyte(x1, x0, sh);
+    auto byte_at = [&](uint32_t i) {
+        return (uint8_t)(__hip_atomic_load(sw + (i >> 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> (8u * (i & 3u)));
+    };
+    if ((uint32_t)lane < head) g[lane] = byte_at((uint32_t)lane);
+    const __amdgpu_buffer_rsrc_t rs = buffer_of(slot, kSpillSlotBytes);
+    const uint32_t ws = head >> 2, bs = head & 3u;   // source word and byte shift, the same for every piece
+    for (uint32_t c = lane; c < nch; c += 64) {
+        const uint32_t s = head + 16u * c;
+        const u32x4 A = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(s & ~15u), 0, kBufStatus);
+        const u32x4 B = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(s & ~15u) + 16, 0, kBufStatus);
+        uint32_t w0, w1, w2, w3, w4;
+        switch (ws) {
+        case 0: w0 = A.x; w1 = A.y; w2 = A.z; w3 = A.w; w4 = B.x; break;
+        case 1: w0 = A.y; w1 = A.z; w2 = A.w; w3 = B.x; w4 = B.y; break;
+        case 2: w0 = A.z; w1 = A.w; w2 = B.x; w3 = B.y; w4 = B.z; break;
+        default: w0 = A.w; w1 = B.x; w2 = B.y; w3 = B.z; w4 = B.w; break;
+        }
+        u32x4 o;
+        o.x = __builtin_amdgcn_alignbyte(w1, w0, bs);
+        o.y = __builtin_amdgcn_alignbyte(w2, w1, bs);
+        o.z = __builtin_amdgcn_alignbyte(w3, w2, bs);
+        o.w = __builtin_amdgcn_alignbyte(w4, w3, bs);
+        stream_store<u32x4>(g + s, o);
     }
-    if ((uint32_t)lane < tail) {
-        const uint32_t s = head + 4u * nw + lane;
-        g[s] = (uint8_t)(word(s >> 2) >> (8 * (s & 3u)));
-    }
+    if ((uint32_t)lane < tail) g[head + 16u * nch + lane] = byte_at(head + 16u * nch + (uint32_t)lane);
 }
 
 // Registers of one incoming stream that travel ahead of the computation.
@@ -514,7 +536,14 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
 
         // ---- this round's tile
         uint32_t run = 0;
-        bool spilled0 = false;
+        // A tile that outgrows its LDS slot goes to the wave's slot of the spill area piece by
+        // piece: whenever the next sub-step would not fit, the whole 16-byte pieces packed so far
+        // are flushed with wide stores and packing goes on at the front of the LDS slot
+        // (`flushed` = tile bytes already in the spill slot, a multiple of 16).  Only a sub-step
+        // that does not fit an empty LDS slot (tiny slots, incompressible data) is packed into
+        // the spill slot directly, byte by byte, and so is the rest of its tile.
+        bool spilled0 = false, direct0 = false;
+        uint32_t flushed = 0;
         if (v0) {
             fetch_headers(r + 1);
             const uint64_t tile_elem0 = (uint64_t)t0 * kTileElems;
@@ -617,18 +646,28 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     analyse8(v, k, a, sb, hd, size, a0);
                     const uint32_t incl = quad_incl_scan_u32(size);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-                    const uint32_t pos = run + incl - size;
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
-                    if (!spilled0 && run + sub_total > slot_cap) {
-                        // the tile outgrows the LDS stage: what is packed so far moves to the spill slot
-                        for (uint32_t i = 4u * lane; i < run; i += 256u)
-                            *reinterpret_cast<uint32_t *>(slot + i) = *reinterpret_cast<const uint32_t *>(stage + i);
+                    if (!direct0 && run - flushed + sub_total > slot_cap) {
+                        const uint32_t local = run - flushed, whole = local & ~15u, rest = local & 15u;
+                        spill_pieces(stage, slot + flushed, whole, lane);
                         spilled0 = true;
+                        if (rest + sub_total > slot_cap) {
+                            // not even an empty slot holds this sub-step: the rest of the tile is packed in place
+                            if ((uint32_t)lane < rest) slot[flushed + whole + (uint32_t)lane] = stage[whole + (uint32_t)lane];
+                            direct0 = true;
+                        } else {
+                            // the bytes beyond the last whole piece move to the front of the slot
+                            const uint8_t moved = (uint32_t)lane < rest ? stage[whole + (uint32_t)lane] : (uint8_t)0;
+                            wave_lds_fence();
+                            if ((uint32_t)lane < rest) stage[lane] = moved;
+                            wave_lds_fence();
+                            flushed += whole;
+                        }
                     }
-                    if (spilled0)
-                        pack8((global_bytes)slot, pos, hd, k, a, sb, a0);
+                    if (direct0)
+                        pack8((global_bytes)slot, run + incl - size, hd, k, a, sb, a0);
                     else
-                        pack8((lds_bytes)stage, pos, hd, k, a, sb, a0);
+                        pack8((lds_bytes)stage, run - flushed + incl - size, hd, k, a, sb, a0);
                     run += sub_total;
                 }
             };
@@ -644,6 +683,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             }
             if constexpr (kEnc) {
                 wave_lds_fence();
+                // the last pieces of a tile that went to the spill slot (rounded up to whole pieces:
+                // the slot has room for them, and what lies beyond the tile's bytes is never read)
+                if (spilled0 && !direct0) spill_pieces(stage, slot + flushed, (run - flushed + 15u) & ~15u, lane);
                 // header bytes of the tile (HomComp/src/GSZ.cu:166)
 #pragma unroll
                 for (int i = lane; i < kTileBlocks; i += 64)
