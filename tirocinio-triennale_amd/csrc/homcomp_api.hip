@@ -182,13 +182,16 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
                 const uint64_t slot_cap = kStage[c][op] / ws->out_slots - 64u;
                 if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) holds = c;
             }
-            // Tiles that no budget holds go through the spill area whatever the choice: the most
-            // waves, then.  The sums are bound by instruction issue and gain more from a third and
-            // fourth workgroup per compute unit than they lose by spilling, so they never take the
-            // large budget by themselves; compress is bound by memory and avoids the spill traffic
-            // where it can.  (Measured on MI355X at 1 GiB, compression ratios 1.6 to 4.4.)
-            cls = holds < 0 ? 0 : holds;
-            if (cls == kStageClasses - 1 && op != hc::kOpCompress) cls = 0;
+            // The sums are bound by instruction issue and gain more from a third and fourth
+            // workgroup per compute unit than they lose by spilling, so they never take the large
+            // budget by themselves; compress is bound by memory and avoids the spill traffic
+            // where it can, and where no budget holds the tiles the medium one is its best
+            // balance between waves and spilled bytes.  (Measured on MI355X at 1 GiB, compression
+            // ratios 1.6 to 4.4.)
+            if (op == hc::kOpCompress)
+                cls = holds < 0 ? 1 : holds;
+            else
+                cls = holds < 0 || holds == kStageClasses - 1 ? 0 : holds;
         }
         if (ws->stage_class >= 0) cls = ws->stage_class;
         p.host_total = &ws->h_mean_tile[op];

@@ -486,7 +486,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     const uint32_t slot_bytes = (p.stage_bytes / (uint32_t)D) & ~15u;
     const uint32_t slot_cap = slot_bytes - 64u;
     uint32_t tot[4] = {0, 0, 0, 0};     // byte totals of the tiles of the previous rounds, newest first
-    bool spl[4] = {false, false, false, false};
+    uint32_t spl[4] = {0, 0, 0, 0};     // how many of their first bytes lie in the spill slot (the rest in the LDS slot)
     uint64_t probe = 0;                // prefix word of the oldest one, requested a round ago
 
     for (int64_t r = 0;; ++r) {
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         if constexpr (kEnc) {
             if (vd) {
                 const uint32_t total_d = D == 2 ? tot[1] : (D == 3 ? tot[2] : tot[3]);
-                const bool spilled_d = D == 2 ? spl[1] : (D == 3 ? spl[2] : spl[3]);
+                const uint32_t spilled_d = D == 2 ? spl[1] : (D == 3 ? spl[2] : spl[3]);
                 // the prefix word travels in lane 0 only: a device-scope load is executed per
                 // lane, so 64 lanes asking for the same word would be 64 requests
                 uint64_t excl = 0;
@@ -527,10 +527,10 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                 excl = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(excl >> 32)) << 32) |
                        (uint32_t)__builtin_amdgcn_readfirstlane((int)excl);
                 uint8_t *dst = p.out_cmp + p.hdr_bytes + excl;
-                if (spilled_d)
-                    copy_out_spill(slot, dst, total_d, lane);
-                else
-                    copy_out<64>(stage, dst, total_d, lane);
+                // the pieces that went to the spill slot, then what stayed in LDS (behind them in the
+                // slot's numbering: LDS position 0 is the tile's byte `spilled_d`)
+                if (spilled_d) copy_out_spill(slot, dst, spilled_d, lane);
+                if (total_d > spilled_d) copy_out<64>(stage, dst + spilled_d, total_d - spilled_d, lane);
             }
         }
 
@@ -539,10 +539,11 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         // A tile that outgrows its LDS slot goes to the wave's slot of the spill area piece by
         // piece: whenever the next sub-step would not fit, the whole 16-byte pieces packed so far
         // are flushed with wide stores and packing goes on at the front of the LDS slot
-        // (`flushed` = tile bytes already in the spill slot, a multiple of 16).  Only a sub-step
+        // (`flushed` = tile bytes already in the spill slot, a multiple of 16); what is in LDS at
+        // the end of the tile stays there until the tile is copied out.  Only a sub-step
         // that does not fit an empty LDS slot (tiny slots, incompressible data) is packed into
         // the spill slot directly, byte by byte, and so is the rest of its tile.
-        bool spilled0 = false, direct0 = false;
+        bool direct0 = false;
         uint32_t flushed = 0;
         if (v0) {
             fetch_headers(r + 1);
@@ -650,7 +651,6 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     if (!direct0 && run - flushed + sub_total > slot_cap) {
                         const uint32_t local = run - flushed, whole = local & ~15u, rest = local & 15u;
                         spill_pieces(stage, slot + flushed, whole, lane);
-                        spilled0 = true;
                         if (rest + sub_total > slot_cap) {
                             // not even an empty slot holds this sub-step: the rest of the tile is packed in place
                             if ((uint32_t)lane < rest) slot[flushed + whole + (uint32_t)lane] = stage[whole + (uint32_t)lane];
@@ -683,9 +683,6 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             }
             if constexpr (kEnc) {
                 wave_lds_fence();
-                // the last pieces of a tile that went to the spill slot (rounded up to whole pieces:
-                // the slot has room for them, and what lies beyond the tile's bytes is never read)
-                if (spilled0 && !direct0) spill_pieces(stage, slot + flushed, (run - flushed + 15u) & ~15u, lane);
                 // header bytes of the tile (HomComp/src/GSZ.cu:166)
 #pragma unroll
                 for (int i = lane; i < kTileBlocks; i += 64)
@@ -696,7 +693,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         if constexpr (kEnc) {
             if (vp && lane == 0) probe = scan_probe(scan, (uint32_t)tp);
             tot[3] = tot[2]; tot[2] = tot[1]; tot[1] = tot[0]; tot[0] = run;
-            spl[3] = spl[2]; spl[2] = spl[1]; spl[1] = spl[0]; spl[0] = spilled0;
+            spl[3] = spl[2]; spl[2] = spl[1]; spl[1] = spl[0]; spl[0] = direct0 ? run : flushed;
         }
     }
 }
