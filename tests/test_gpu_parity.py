@@ -277,6 +277,39 @@ def test_offsets_prepass_sizes(pkg, cuda, orc, gen, tiles, offset):
         g.close()
 
 
+def mixed_field(gen, rng, n):
+    """Segments of the three generators at scales from 1e-3 to 1e3, with runs of exact zeros: plane
+    counts change from block to block and from step to step inside one tile."""
+    out = np.zeros(n, np.float32)
+    i = 0
+    while i < n:
+        m = int(min(n - i, rng.integers(1, 6000)))
+        kind = int(rng.integers(0, 4))
+        if kind < 3:
+            seg = (gen.smooth_np, gen.gradient_like_np, gen.uniform_np)[kind](max(m, 32), int(rng.integers(1, 1 << 30)))[:m]
+            out[i:i + m] = seg * np.float32(10.0 ** rng.uniform(-3, 3))
+        i += m
+    return out
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_mixtures(gpu, orc, gen, seed):
+    """Random lengths, error bounds and mixtures of data kinds, every operation against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(1, 400000))
+    a, b = mixed_field(gen, rng, n), mixed_field(gen, rng, n)
+    eb = np.float32(10.0 ** rng.uniform(-5, 0))
+    sa, sb = orc.compress(a, eb), orc.compress(b, eb)
+    assert_stream_equal(gpu.compress(a, eb), sa, "compress")
+    want = orc.hom_sum_f32(sa, b, eb)
+    assert_stream_equal(gpu.hom_sum_f32(sa, b, eb), want, "hom_sum_f32")
+    assert_stream_equal(gpu.hom_add(sa, sb, n), want, "hom_add")
+    qp = orc.quant_predict(b, eb)
+    assert_stream_equal(gpu.hom_sum_i32(sa, qp), orc.hom_sum_i32(sa, qp), "hom_sum_i32")
+    dec = gpu.decompress(want, n, eb)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(want, n, eb).view(np.uint32))
+
+
 def test_value_range(gpu, orc, gen, pkg):
     for kind, n in (("smooth", 1 << 20), ("uniform", 12345), ("gradient_like", 7)):
         x = make(gen, kind, n, seed=4)
