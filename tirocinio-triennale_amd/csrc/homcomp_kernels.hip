@@ -725,11 +725,15 @@ __device__ __forceinline__ uint32_t wg_reduce_u32(uint32_t v, uint32_t *s_tmp)
     return t;
 }
 
+// A stream of at most one block of tiles (4 MiB of values) gets its offsets from k_in_totals
+// itself (`ofs` not null, one workgroup): the second launch would be a fifth of such a call.
 __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ hdr, uint32_t n_tiles,
                                                    uint32_t *__restrict__ totals,
-                                                   uint32_t *__restrict__ block_sums)
+                                                   uint32_t *__restrict__ block_sums,
+                                                   uint64_t base, uint64_t *__restrict__ ofs)
 {
     __shared__ uint32_t s_tmp[4];
+    __shared__ uint32_t s_tot[kOfsBlockTiles];
     uint32_t acc = 0;
     constexpr uint32_t kPieces = kTileBlocks / 16;            // 16-byte header pieces (lanes) per tile
     constexpr uint32_t kPasses = kOfsBlockTiles * kPieces / 256;
@@ -769,10 +773,26 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
         sum += dpp_u32<kDppXor1>(sum);
         sum += dpp_u32<kDppXor2>(sum);
         sum += dpp_u32<kDppRowHalfMirror>(sum);   // the other quad of the eight
-        if (tile < n_tiles && (threadIdx.x & (kPieces - 1)) == 0) totals[tile] = sum;
+        if ((threadIdx.x & (kPieces - 1)) == 0) {
+            if (tile < n_tiles) totals[tile] = sum;
+            s_tot[tile % kOfsBlockTiles] = sum;   // 0 beyond the last tile
+        }
     }
-    const uint32_t block_total = wg_reduce_u32(acc, s_tmp);
+    const uint32_t block_total = wg_reduce_u32(acc, s_tmp);   // with a barrier: s_tot is complete
     if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total;
+    if (ofs == nullptr) return;
+    // one block of tiles: its offsets right away, as k_in_offsets below would compute them
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t mine = s_tot[threadIdx.x];
+    const uint32_t incl = wave_incl_scan_u32(mine, lane);
+    if (lane == 63) s_tmp[wave] = incl;
+    __syncthreads();
+    uint32_t earlier = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        if (q < wave) earlier += s_tmp[q];
+    if (threadIdx.x < n_tiles) ofs[threadIdx.x] = base + earlier + (incl - mine);
+    if (threadIdx.x == 0) ofs[n_tiles] = base + block_total;   // the end of the payload
 }
 
 __global__ __launch_bounds__(256) void k_in_offsets(const uint32_t *__restrict__ totals,
@@ -985,7 +1005,12 @@ hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base
                              uint32_t *block_sums, uint64_t *ofs, hipStream_t s)
 {
     const uint32_t blocks = (n_tiles + kOfsBlockTiles - 1) / kOfsBlockTiles;
-    hipLaunchKernelGGL(k_in_totals, dim3(blocks), dim3(256), 0, s, hdr, n_tiles, totals, block_sums);
+    if (blocks == 1) {
+        hipLaunchKernelGGL(k_in_totals, dim3(1), dim3(256), 0, s, hdr, n_tiles, totals, block_sums, base, ofs);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(k_in_totals, dim3(blocks), dim3(256), 0, s, hdr, n_tiles, totals, block_sums, (uint64_t)0,
+                       (uint64_t *)nullptr);
     hipLaunchKernelGGL(k_in_offsets, dim3(blocks), dim3(256), 0, s, totals, block_sums, n_tiles, base, ofs);
     return hipGetLastError();
 }
