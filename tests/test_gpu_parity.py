@@ -440,3 +440,58 @@ def test_two_streams_do_not_overlap_their_scans(pkg, cuda, orc, gen):
         assert_stream_equal(out1[1][:L1].cpu().numpy(), want_b, "compress on stream 1")
         assert_stream_equal(out1[0][:want_a.size].cpu().numpy(), want_a, "compress on stream 1 (even calls)")
         assert_stream_equal(out2[1][:L2].cpu().numpy(), want_sum, "hom_sum_f32 on stream 2")
+
+
+def test_graph_replay(pkg, cuda, orc, gen):
+    """compress, hom_sum_f32 and decompress captured into one HIP graph (no call allocates or
+    blocks when the lengths go to device words) and replayed with new operand contents, with
+    eager calls on the same workspace between the replays: every replay gives the oracle's bytes.
+    Incoming sizes are fixed at capture time, so the graph states the buffer capacity; a
+    well-formed stream decodes the same under any stated size that covers it."""
+    torch = cuda
+    orc.set_threads(16)
+    n = (1 << 20) + 4099
+    eb = np.float32(8e-4)
+    cap = pkg.max_stream_bytes(n)
+    x = torch.empty(n, dtype=torch.float32, device="cuda")
+    y = torch.empty(n, dtype=torch.float32, device="cuda")
+    ca = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    cs = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    other = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    dec = torch.empty(n, dtype=torch.float32, device="cuda")
+    lens = torch.zeros(2, dtype=torch.int64, device="cuda")
+    la, ls = lens[0:1], lens[1:2]
+    with pkg.Workspace(n) as ws:
+        def work():
+            ws.compress(x, float(eb), ca, stream_len=la)
+            ws.hom_sum_f32(ca, cap, y, float(eb), cs, stream_len=ls)
+            ws.decompress(cs, cap, n, float(eb), dec)
+
+        x.copy_(torch.from_numpy(gen.smooth_np(n, 80)))
+        y.copy_(torch.from_numpy(gen.smooth_np(n, 81)))
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            work()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            work()
+        for i, (mk_x, mk_y) in enumerate([(gen.smooth_np, gen.gradient_like_np), (gen.uniform_np, gen.smooth_np),
+                                          (gen.smooth_np, gen.smooth_np), (gen.gradient_like_np, gen.uniform_np)]):
+            hx, hy = mk_x(n, 90 + i), mk_y(n, 95 + i)
+            x.copy_(torch.from_numpy(hx))
+            y.copy_(torch.from_numpy(hy))
+            graph.replay()
+            torch.cuda.synchronize()
+            want_a = orc.compress(hx, eb)
+            want_s = orc.hom_sum_f32(want_a, hy, eb)
+            l1, l2 = (int(v) for v in lens.cpu())
+            assert l1 == want_a.size and l2 == want_s.size, f"replay {i}: lengths {l1}, {l2}"
+            assert_stream_equal(ca[:l1].cpu().numpy(), want_a, f"replay {i}: compress")
+            assert_stream_equal(cs[:l2].cpu().numpy(), want_s, f"replay {i}: hom_sum_f32")
+            assert np.array_equal(dec.cpu().numpy().view(np.uint32), orc.decompress(want_s, n, eb).view(np.uint32))
+            # eager work of the program between the replays, on the same workspace
+            ws.compress(y, float(eb), other)
+            assert ws.last_size() == orc.compress(hy, eb).size

@@ -127,8 +127,8 @@ constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
 // its whole grid resident (the scan's waits), and two such grids from different streams can each
 // end up half resident, every wave waiting for workgroups that cannot start: both calls would
 // run into the bound of their waits.  So a launch on another stream than the device's previous
-// one first waits (on the GPU, not on the host) for an event recorded on that stream.  A stream under capture is
-// left alone: its graph orders the launches it contains.
+// one first waits (on the GPU, not on the host) for an event recorded on that stream.  A stream
+// under capture is left alone: its graph orders the launches it contains.
 struct DeviceChain {
     std::mutex mu;
     hipEvent_t done = nullptr;
@@ -142,7 +142,13 @@ int chained_launch(homcomp_workspace *ws, int op, const hc::TileParams &p, uint3
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
     if (capturing || ws->device < 0 || ws->device >= 64) {
-        if (capturing) (void)hipGetLastError();
+        if (capturing) {
+            (void)hipGetLastError();
+            // A captured launch is replayed with the epoch it was captured with, so the scan words
+            // of the previous replay would read as this call's: the graph clears them first (with
+            // a kernel; memset nodes are avoided in graphs).
+            if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s))) return HOMCOMP_ERR_HIP;
+        }
         return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
     DeviceChain &c = g_chain[ws->device];
