@@ -57,6 +57,7 @@ struct homcomp_workspace {
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint8_t *d_spill;         // spill slots: four worst-case tiles per data wave
     uint32_t out_slots;       // deferral depth of packed tiles (2..4)
+    uint32_t sliced;          // HOMCOMP_SLICED=0 switches the bit-plane path of stream (+) stream off
     int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
 };
 
@@ -120,8 +121,8 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 constexpr int kStageClasses = 3;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
-    {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4544 + 64)},
-    {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7680 + 64)}};
+    {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (3888 + 64)},
+    {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7216 + 64)}};
 
 // The stream-producing kernels of this process never overlap on a device.  Each of them needs
 // its whole grid resident (the scan's waits), and two such grids from different streams can each
@@ -176,6 +177,7 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
 {
     p.spill = ws->d_spill;
     p.out_slots = ws->out_slots;
+    p.sliced = ws->sliced;
     int cls = kStageClasses - 1;
     if (op == hc::kOpDecompress) {
         cls = 0;
@@ -325,6 +327,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (std::strcmp(e, "medium") == 0) ws->stage_class = 1;
         if (std::strcmp(e, "large") == 0) ws->stage_class = 2;
     }
+    ws->sliced = 1;
+    if (const char *e = std::getenv("HOMCOMP_SLICED")) ws->sliced = std::strtol(e, nullptr, 10) != 0;
     ws->out_slots = 2;
     if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
         const long v = std::strtol(e, nullptr, 10);

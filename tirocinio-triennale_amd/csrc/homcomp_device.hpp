@@ -420,6 +420,142 @@ __device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0,
     }
 }
 
+// ---------------------------------------------------------------- sums in the bit-plane domain
+//
+// A plane of a block is one 32-bit word of the stream, so with one lane per block a single
+// instruction handles a plane of all 32 elements: stream (+) stream needs no transposition at
+// all.  Blocks of at most kSlicedMaxF planes are read as words (outlier bytes, sign word,
+// planes), turned into two's complement plane by plane (invert where the sign bit is set, ripple
+// the +1), added with a ripple of full adders, and turned back into sign and magnitude; the
+// result is at most kSlicedMaxF + 1 bits wide.  Element 0 is kept out of the planes and handled
+// as a scalar: in outlier mode its magnitude is the outlier (HomComp/src/GSZ.cu:913-917,
+// 1005-1006), which has up to 32 bits.  In a word of the stream, byte k bit 7-m is element
+// 8k+m, so element 0 is bit 7; sums of deltas need no order of the elements, and the words go
+// out as they came in.
+constexpr uint32_t kSlicedMaxF = 6;
+constexpr int kSlicedOutPlanes = kSlicedMaxF + 2;   // plain mode can take element 0 one plane further
+
+typedef uint32_t __attribute__((aligned(1))) u32_unaligned;
+__device__ __forceinline__ uint32_t load_u32_any(const uint8_t *p) { return *reinterpret_cast<const u32_unaligned *>(p); }
+__device__ __forceinline__ void store_u32_any(lds_bytes p, uint32_t v)
+{
+    *(__attribute__((address_space(3))) u32_unaligned *)p = v;
+}
+
+struct SlicedIn {
+    uint32_t a0, sign, ob, pl[kSlicedMaxF];
+};
+
+// The lane's block of an incoming stream from the LDS stage (`p0` = the block's first byte);
+// digest 0 (no payload, or not to be read) gives a block of zeros.
+__device__ __forceinline__ void sliced_read(const uint8_t *stage, uint32_t p0, uint32_t digest, SlicedIn &b)
+{
+    const uint32_t F = digest & 0x1fu;
+    b.ob = digest >> 5;
+    const uint32_t first = load_u32_any(stage + p0);
+    const uint32_t low_bytes = ~(0xffffff00u << ((8u * (b.ob - 1u)) & 31u));   // ob = 1..4
+    b.a0 = b.ob ? first & low_bytes : 0u;
+    const uint32_t sign = load_u32_any(stage + p0 + b.ob);
+    b.sign = digest ? sign : 0u;
+#pragma unroll
+    for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+        const uint32_t w = load_u32_any(stage + p0 + b.ob + 4u + 4u * q);
+        b.pl[q] = q < F ? w : 0u;
+    }
+}
+
+struct SlicedOut {
+    uint32_t hdr, size, ob, F, a0, sign, m[kSlicedOutPlanes];
+};
+
+// delta_out = delta_A + delta_B for the lane's block, and the block's rate selection
+// (HomComp/src/GSZ.cu:151-167).
+__device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B, SlicedOut &o)
+{
+    constexpr uint32_t E = 0x80u;   // element 0
+    // ---- element 0: plane bits in plain mode, the outlier in outlier mode
+    uint32_t m0A = A.a0, m0B = B.a0;
+    {
+        uint32_t anyA = 0, anyB = 0;
+#pragma unroll
+        for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+            anyA |= A.pl[q];
+            anyB |= B.pl[q];
+        }
+        const bool gatherA = A.ob == 0u && (anyA & E), gatherB = B.ob == 0u && (anyB & E);
+        if (__builtin_amdgcn_ballot_w64(gatherA || gatherB) != 0) {   // wave-uniform; rare where outlier mode prevails
+            uint32_t gA = 0, gB = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+                gA |= ((A.pl[q] >> 7) & 1u) << q;
+                gB |= ((B.pl[q] >> 7) & 1u) << q;
+            }
+            if (A.ob == 0u) m0A = gA;
+            if (B.ob == 0u) m0B = gB;
+        }
+    }
+    const uint32_t v0A = (A.sign & E) ? 0u - m0A : m0A, v0B = (B.sign & E) ? 0u - m0B : m0B;
+    const uint32_t s0 = v0A + v0B;   // wrapping, as the reference's int
+    const int32_t s0neg = (int32_t)(0u - s0);
+    o.a0 = (uint32_t)((int32_t)s0 > s0neg ? (int32_t)s0 : s0neg);   // |s0| (0x80000000 stays)
+    // ---- elements 1..31, plane by plane
+    const uint32_t SA = A.sign & ~E, SB = B.sign & ~E;
+    uint32_t cA = SA, cB = SB, carry = 0, r[kSlicedMaxF + 2];
+#pragma unroll
+    for (uint32_t q = 0; q < kSlicedMaxF + 2; ++q) {
+        const uint32_t tA = (q < kSlicedMaxF ? A.pl[q] & ~E : 0u) ^ SA;
+        const uint32_t tB = (q < kSlicedMaxF ? B.pl[q] & ~E : 0u) ^ SB;
+        const uint32_t xA = tA ^ cA, xB = tB ^ cB;
+        cA &= tA;
+        cB &= tB;
+        r[q] = xA ^ xB ^ carry;
+        carry = (xA & xB) | (carry & (xA ^ xB));
+    }
+    const uint32_t SR = r[kSlicedMaxF + 1];   // the sign plane: the sums fit kSlicedMaxF + 1 bits
+    uint32_t c = SR, nz = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < kSlicedOutPlanes; ++q) o.m[q] = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < kSlicedMaxF + 1; ++q) {
+        const uint32_t t = r[q] ^ SR;
+        o.m[q] = t ^ c;
+        c &= t;
+        nz |= (o.m[q] ? 1u : 0u) << q;
+    }
+    // ---- rate selection
+    const uint32_t fr2 = bit_num(nz);                      // elements 1..31   (:153)
+    const uint32_t b0 = bit_num(o.a0);
+    uint32_t fr1 = b0 > fr2 ? b0 : fr2;                    // all 32 elements  (:152)
+    if (fr1 > 31u) fr1 = 31u;
+    const uint32_t ob = (b0 + 7u) >> 3;                    // :154
+    const uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;         // :156
+    const uint32_t sz2 = 4u + 4u * fr2 + ob;               // :157
+    const bool plain = sz1 <= sz2;                         // :158-164
+    o.hdr = plain ? fr1 : fr2 | 0x80u | ((ob - 1u) << 5);
+    o.size = plain ? sz1 : sz2;
+    o.F = plain ? fr1 : fr2;
+    o.ob = plain ? 0u : ob;
+    o.sign = SR | (((int32_t)s0 < 0) ? E : 0u);
+    // plain mode: element 0 goes back into the planes (it has at most one plane more than the rest)
+    const uint32_t ins = plain ? o.a0 : 0u;
+    if (__builtin_amdgcn_ballot_w64(ins != 0u) != 0) {
+#pragma unroll
+        for (uint32_t q = 0; q < kSlicedOutPlanes; ++q) o.m[q] |= ((ins >> q) & 1u) << 7;
+    }
+}
+
+// The block's payload at `pos` of the stage: outlier bytes (a whole word is stored; what it
+// writes beyond them is overwritten by the sign word), sign word, planes.
+__device__ __forceinline__ void sliced_write(lds_bytes stage, uint32_t pos, const SlicedOut &o)
+{
+    if (o.hdr == 0u) return;
+    if (o.ob) store_u32_any(stage + pos, o.a0);
+    store_u32_any(stage + pos + o.ob, o.sign);
+#pragma unroll
+    for (uint32_t q = 0; q < (uint32_t)kSlicedOutPlanes; ++q)
+        if (q < o.F) store_u32_any(stage + pos + o.ob + 4u + 4u * q, o.m[q]);
+}
+
 // ---------------------------------------------------------------- output-offset scan
 //
 // The byte offset of a tile's payload in the outgoing stream is an exclusive prefix sum over

@@ -243,6 +243,9 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
 // area and is copied out from there.
 constexpr int kSub = kTileBlocks / 16;
 constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
+// stream (+) stream stages whole tiles of few planes for the sums in the bit-plane domain
+constexpr int kInStageTile = 3584;
+constexpr int kInStageTileSlack = 64;   // alignment shift of the range, words read beyond the last block
 
 template <int LOCAL>
 struct SubRegs {
@@ -346,7 +349,9 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     extern __shared__ __align__(16) uint8_t s_dyn[];
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
     // one stage per wave: the incoming streams of a sub-step are decoded one after the other
-    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInStage : 16];
+    // stream (+) stream as a sum in the bit-plane domain, tile by tile where the tiles allow it
+    constexpr bool kSliced = kEnc && NIN == 2 && LOCAL == kLocalNone;
+    __shared__ __align__(16) uint8_t s_in[kW][kSliced ? kInStageTile : (NIN > 0 ? kInStage : 16)];
     __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
     __shared__ __align__(4) uint8_t s_hdr_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 4];
     __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512];     // decoder: exchange of the lanes' output pieces
@@ -379,6 +384,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // bytes of the stream from the tile's payload start to its stated end, saturated to 32 bits:
     // everything inside a tile is 32-bit arithmetic against these
     uint32_t room_ctx0[kIn], room_ctx1[kIn];
+    bool few_ctx0[kIn], few_ctx1[kIn];   // kSliced: the tile has few planes per block and fits the stage as a whole
     auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             int64_t t = tile_of(r);
@@ -414,12 +420,20 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     const uint32_t d0 = z0 != 0u && o0 < room ? header_digest(h0) : 0u;
                     const uint32_t d1 = z1 != 0u && o1 < room ? header_digest(h1) : 0u;
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
+                    bool few = false;
+                    if constexpr (kSliced) {
+                        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+                        few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0 &&
+                              total + kInStageTileSlack <= (uint32_t)kInStageTile;
+                    }
                     if (b) {
                         start_ctx1[c] = start_next[c];
                         room_ctx1[c] = room;
+                        few_ctx1[c] = few;
                     } else {
                         start_ctx0[c] = start_next[c];
                         room_ctx0[c] = room;
+                        few_ctx0[c] = few;
                     }
                 }
                 wave_lds_fence();
@@ -548,6 +562,98 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         if (v0) {
             fetch_headers(r + 1);
             const uint64_t tile_elem0 = (uint64_t)t0 * kTileElems;
+            // room in the LDS slot for the next `bytes` of the tile (see above); false: they are to
+            // be packed into the spill slot in place
+            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {
+                if (!direct0 && run - flushed + bytes > slot_cap) {
+                    const uint32_t local = run - flushed, whole = local & ~15u, rest = local & 15u;
+                    spill_pieces(stage, slot + flushed, whole, lane);
+                    if (rest + bytes > slot_cap) {
+                        // not even an empty slot holds this much: the rest of the tile is packed in place
+                        if ((uint32_t)lane < rest) slot[flushed + whole + (uint32_t)lane] = stage[whole + (uint32_t)lane];
+                        direct0 = true;
+                    } else {
+                        // the bytes beyond the last whole piece move to the front of the slot
+                        const uint8_t moved = (uint32_t)lane < rest ? stage[whole + (uint32_t)lane] : (uint8_t)0;
+                        wave_lds_fence();
+                        if ((uint32_t)lane < rest) stage[lane] = moved;
+                        wave_lds_fence();
+                        flushed += whole;
+                    }
+                }
+                return !direct0;
+            };
+            bool sliced_tile = false;
+            if constexpr (kSliced) {
+                // 32 blocks of at most 40 bytes must fit an empty slot (they are written at once)
+                sliced_tile = p.sliced && slot_cap >= 32u * 40u + 16u &&
+                              (buf ? few_ctx1[0] && few_ctx1[1] : few_ctx0[0] && few_ctx0[1]);
+            }
+            if (sliced_tile) {
+                if constexpr (kSliced) {
+                    // ---- the whole tile in the bit-plane domain: lane L owns blocks L and 64 + L
+                    uint8_t *st = s_in[wave];
+                    SlicedIn A[2];
+                    uint32_t shift_c[2];
+                    u32x4 piece[2][kInStageTile / 1024 + 1];
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        const uint32_t total = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][kSub]);
+                        const uint32_t room = buf ? room_ctx1[c] : room_ctx0[c];
+                        const uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
+                        const uint32_t end = total < lim ? total : lim;
+                        const uintptr_t g0 = (uintptr_t)p.in[c] + (buf ? start_ctx1[c] : start_ctx0[c]);
+                        const uintptr_t ga = g0 & ~(uintptr_t)15;
+                        shift_c[c] = (uint32_t)(g0 - ga);
+                        const uint32_t nbytes = end ? shift_c[c] + end : 0u;
+                        const __amdgpu_buffer_rsrc_t rs = buffer_of(reinterpret_cast<const void *>(ga), (nbytes + 15u) & ~15u);
+#pragma unroll
+                        for (int i = 0; i < kInStageTile / 1024 + 1; ++i)
+                            piece[c][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (lane + 64 * i) * 16, 0, kBufCached);
+                    }
+                    SlicedOut out;
+                    auto stage_stream = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int i = 0; i < kInStageTile / 1024 + 1; ++i)
+                            if ((lane + 64 * i) * 16 < kInStageTile)
+                                *reinterpret_cast<u32x4 *>(st + (lane + 64 * i) * 16) = piece[c][i];
+                        wave_lds_fence();
+                    };
+                    auto read_block = [&](int c, int half, SlicedIn &blk) __attribute__((always_inline)) {
+                        const int b = half * 64 + lane;
+                        sliced_read(st, shift_c[c] + s_ofs_in[wave][c][buf][b], s_hdr_in[wave][c][buf][b], blk);
+                    };
+                    stage_stream(0);
+                    read_block(0, 0, A[0]);
+                    read_block(0, 1, A[1]);
+                    wave_lds_fence();
+                    stage_stream(1);
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        SlicedIn B;
+                        read_block(1, half, B);
+                        sliced_add(A[half], B, out);
+                        s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
+                        const uint32_t incl = wave_incl_scan_u32(out.size, lane);
+                        const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
+                        const uint32_t all64 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+                        // two writes of 32 blocks each, so that what is written at once fits an empty slot
+#pragma unroll
+                        for (int q = 0; q < 2; ++q) {
+                            const uint32_t bytes = q ? all64 - first32 : first32;
+                            make_room(bytes);   // always true here: 32 blocks fit an empty slot
+                            const uint32_t pos = run - flushed + (incl - out.size) - (q ? first32 : 0u);
+                            if ((lane >> 5) == q) sliced_write((lds_bytes)stage, pos, out);
+                            run += bytes;
+                        }
+                    }
+                    wave_lds_fence();
+                    // the next tile's block offsets and first requests, as the sub-steps below leave them
+                    prepare(r + 1, buf ^ 1);
+#pragma unroll
+                    for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j]);
+                }
+            } else {
             // sub-step s of this tile; (r2, b2, s2) is the sub-step the freed registers are requested for
             auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2) __attribute__((always_inline)) {
                 // the blocks' digests and offsets first: nothing in the sub-step writes them, and
@@ -648,22 +754,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     const uint32_t incl = quad_incl_scan_u32(size);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
-                    if (!direct0 && run - flushed + sub_total > slot_cap) {
-                        const uint32_t local = run - flushed, whole = local & ~15u, rest = local & 15u;
-                        spill_pieces(stage, slot + flushed, whole, lane);
-                        if (rest + sub_total > slot_cap) {
-                            // not even an empty slot holds this sub-step: the rest of the tile is packed in place
-                            if ((uint32_t)lane < rest) slot[flushed + whole + (uint32_t)lane] = stage[whole + (uint32_t)lane];
-                            direct0 = true;
-                        } else {
-                            // the bytes beyond the last whole piece move to the front of the slot
-                            const uint8_t moved = (uint32_t)lane < rest ? stage[whole + (uint32_t)lane] : (uint8_t)0;
-                            wave_lds_fence();
-                            if ((uint32_t)lane < rest) stage[lane] = moved;
-                            wave_lds_fence();
-                            flushed += whole;
-                        }
-                    }
+                    make_room(sub_total);
                     if (direct0)
                         pack8((global_bytes)slot, run + incl - size, hd, k, a, sb, a0);
                     else
@@ -680,6 +771,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                 const int s2 = s + kDepth - wrap * kSub;
 #pragma unroll
                 for (int j = 0; j < kDepth; ++j) sub(s + j, loc[j], in[j], r + wrap, buf ^ wrap, s2 + j);
+            }
             }
             if constexpr (kEnc) {
                 wave_lds_fence();
