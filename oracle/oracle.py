@@ -264,12 +264,13 @@ def hom_sum_i32(cmp_in, local_delta, cmp_in_size: int | None = None) -> np.ndarr
     return out[:L.value].copy()
 
 
-def hom_add(cmp_a, cmp_b, n: int) -> np.ndarray:
+def hom_add(cmp_a, cmp_b, n: int, size_a: int | None = None, size_b: int | None = None) -> np.ndarray:
     a, b = _u8(cmp_a), _u8(cmp_b)
     ba, bb = _padded_stream(a, n), _padded_stream(b, n)
     out = np.zeros(max_stream_bytes(n), np.uint8)
     L = C.c_size_t()
-    rc = lib().hco_hom_add(_p(ba, C.c_uint8), a.size, _p(bb, C.c_uint8), b.size, n,
+    rc = lib().hco_hom_add(_p(ba, C.c_uint8), a.size if size_a is None else size_a,
+                           _p(bb, C.c_uint8), b.size if size_b is None else size_b, n,
                            _p(out, C.c_uint8), C.byref(L))
     assert rc == 0
     return out[:L.value].copy()

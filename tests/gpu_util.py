@@ -69,10 +69,11 @@ class Gpu:
         L = self.ws.last_size()
         return out[:L].cpu().numpy()
 
-    def hom_add(self, a: np.ndarray, b: np.ndarray, n: int) -> np.ndarray:
-        ba, bb = self.put_stream(a, n), self.put_stream(b, n, offset=3)
+    def hom_add(self, a: np.ndarray, b: np.ndarray, n: int, size_a: int | None = None,
+                size_b: int | None = None, offset: int = 0) -> np.ndarray:
+        ba, bb = self.put_stream(a, n, offset=offset), self.put_stream(b, n, offset=3)
         out = self.stream_buf(n)
-        self.ws.hom_add(ba, a.size, bb, b.size, n, out)
+        self.ws.hom_add(ba, a.size if size_a is None else size_a, bb, b.size if size_b is None else size_b, n, out)
         L = self.ws.last_size()
         return out[:L].cpu().numpy()
 

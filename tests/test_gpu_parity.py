@@ -178,6 +178,49 @@ def test_few_planes_per_step(gpu, orc):
         assert np.array_equal(dec.view(np.uint32), orc.decompress(s1, n, 0.5).view(np.uint32)), f"decompress #{trial}"
 
 
+def test_sums_in_the_bit_plane_domain(gpu, orc):
+    """stream (+) stream on tiles whose blocks have at most six planes is computed plane by plane,
+    a block per lane, element 0 beside it as a scalar.  Crafted deltas: every plane count 0..6 on
+    both sides (carries into the seventh and eighth plane), plain and outlier mode on either side
+    and in the result, outliers of 1..4 bytes with both signs, first elements that cancel,
+    whole tiles of empty blocks, and one block of seven planes that sends its tile down the
+    general path between tiles that take the fast one."""
+    rng = np.random.default_rng(23)
+    n = 1 << 17
+    nb = n // 32
+
+    def craft(seed_shift):
+        d = np.zeros((nb, 32), np.int64)
+        for b in range(nb):
+            F = int(rng.integers(0, 7))
+            if F:
+                d[b] = rng.integers(0, 1 << F, 32) * (rng.integers(0, 2, 32) * 2 - 1)
+            kind = int(rng.integers(0, 6))
+            if kind == 0:      # outlier of 1..4 bytes in front
+                d[b, 0] = int(rng.integers(1, 1 << int(rng.integers(1, 32)))) * int(rng.integers(0, 2) * 2 - 1)
+            elif kind == 1:    # only the first element
+                d[b, 1:] = 0
+            elif kind == 2:    # empty block
+                d[b] = 0
+        d[(3 * 128 + seed_shift) % nb:(3 * 128 + seed_shift) % nb + 128] = 0          # a tile of empty blocks
+        d[5 * 128 + 17, 9] = 64 + seed_shift                                          # seven planes: general path
+        return d
+
+    d1, d2 = craft(0), craft(1)
+    d2[::7, 0] = -d1[::7, 0]                       # first elements that cancel
+    d2[1::11] = -d1[1::11]                         # whole blocks that cancel
+    d1, d2 = d1.reshape(-1).astype(np.int32), d2.reshape(-1).astype(np.int32)
+    s1, s2 = orc.encode_deltas(d1), orc.encode_deltas(d2)
+    want = orc.encode_deltas(d1 + d2)
+    assert_stream_equal(orc.hom_add(s1, s2, n), want, "oracle: hom_add of crafted streams")
+    assert_stream_equal(gpu.hom_add(s1, s2, n), want, "hom_add")
+    assert_stream_equal(gpu.hom_add(s2, s1, n), want, "hom_add, operands swapped")
+    # unaligned stream pointers and a stated size that cuts the second stream short
+    assert_stream_equal(gpu.hom_add(s1, s2, n, offset=3), want, "hom_add, unaligned")
+    cut = orc.header_bytes(n) + (s2.size - orc.header_bytes(n)) // 2 + 5
+    assert_stream_equal(gpu.hom_add(s1, s2, n, size_b=cut), orc.hom_add(s1, s2, n, size_b=cut), "hom_add, truncated")
+
+
 def test_zero_incoming_blocks(gpu, orc, gen):
     """Incoming blocks with a zero header contribute nothing (the reference leaves stale
     registers there, HomComp/src/homcomp.cu:3086,3149); the local data must still be added."""
