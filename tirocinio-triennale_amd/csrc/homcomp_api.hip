@@ -112,12 +112,12 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 
 // LDS stage per data wave (two deferred tiles by default), in three budgets that let 4, 3 and 2
 // workgroups share a compute unit (with the LDS the kernels hold besides: 0.6 KiB for compress,
-// 12.5 KiB with one incoming stream, 15.8 KiB with two).  The slots hold tiles of streams
+// 12.5 KiB with one incoming stream, 21.1 KiB with two).  The slots hold tiles of streams
 // compressed about 4.6x / 2.9x / 2x or better for compress, 6x / 3.7x / 2x for the sums with one
-// incoming stream and 9x / 4x / 2.1x with two.  A tile beyond its slot still works (it goes
+// incoming stream and 9x / 4.8x / 2.6x with two.  A tile beyond its slot still works (it goes
 // through the spill area), so the choice below is a performance heuristic, never a correctness
 // matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
-// fits a compute unit, which is slower than spilling: its largest slots are 7.5 KiB.)
+// fits a compute unit, which is slower than spilling: its largest slots are 7 KiB.)
 constexpr int kStageClasses = 3;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
