@@ -221,6 +221,30 @@ def test_sums_in_the_bit_plane_domain(gpu, orc):
     assert_stream_equal(gpu.hom_add(s1, s2, n, size_b=cut), orc.hom_add(s1, s2, n, size_b=cut), "hom_add, truncated")
 
 
+@pytest.mark.parametrize("max_planes", [6, 31])
+def test_arbitrary_payload_bytes(gpu, orc, max_planes):
+    """Headers of a well-formed stream over payloads of random bytes: every byte pattern decodes to
+    something (sign bits on zero magnitudes, plane bits of element 0 set in outlier mode, where
+    the outlier replaces them, HomComp/src/GSZ.cu:1005-1006), and the GPU must read it as the
+    oracle does, in stream (+) stream (bit-plane path with at most six planes, general path
+    with up to 31), in stream (+) int32 deltas and in decompress."""
+    rng = np.random.default_rng(31 + max_planes)
+    n = 1 << 16
+    caps = np.full(n // 512, max_planes)
+    streams = []
+    for _ in range(2):
+        st = orc.encode_deltas(rand_deltas(rng, n // 32, caps)).copy()
+        hb = orc.header_bytes(n)
+        st[hb:] = rng.integers(0, 256, st.size - hb, dtype=np.uint8)
+        streams.append(st)
+    a, b = streams
+    assert_stream_equal(gpu.hom_add(a, b, n), orc.hom_add(a, b, n), "hom_add")
+    d = rand_deltas(rng, n // 32, caps)
+    assert_stream_equal(gpu.hom_sum_i32(a, d), orc.hom_sum_i32(a, d), "hom_sum_i32")
+    dec = gpu.decompress(a, n, 0.5)
+    assert np.array_equal(dec.view(np.uint32), orc.decompress(a, n, 0.5).view(np.uint32))
+
+
 def test_zero_incoming_blocks(gpu, orc, gen):
     """Incoming blocks with a zero header contribute nothing (the reference leaves stale
     registers there, HomComp/src/homcomp.cu:3086,3149); the local data must still be added."""
