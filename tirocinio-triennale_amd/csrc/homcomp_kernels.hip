@@ -244,8 +244,7 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
 constexpr int kSub = kTileBlocks / 16;
 constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
 // stream (+) stream stages whole tiles of few planes for the sums in the bit-plane domain
-constexpr int kInStageTile = 3584;
-constexpr int kInStageTileSlack = 64;   // alignment shift of the range, words read beyond the last block
+constexpr int kInStageTile = 3584;   // half a tile of such blocks (three 1 KiB pieces) and the words read beyond its last block
 
 template <int LOCAL>
 struct SubRegs {
@@ -384,7 +383,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // bytes of the stream from the tile's payload start to its stated end, saturated to 32 bits:
     // everything inside a tile is 32-bit arithmetic against these
     uint32_t room_ctx0[kIn], room_ctx1[kIn];
-    bool few_ctx0[kIn], few_ctx1[kIn];   // kSliced: the tile has few planes per block and fits the stage as a whole
+    bool few_ctx0[kIn], few_ctx1[kIn];   // kSliced: no block of the tile has more than kSlicedMaxF planes
     auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             int64_t t = tile_of(r);
@@ -422,9 +421,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
                     bool few = false;
                     if constexpr (kSliced) {
-                        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-                        few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0 &&
-                              total + kInStageTileSlack <= (uint32_t)kInStageTile;
+                        few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0;
                     }
                     if (b) {
                         start_ctx1[c] = start_next[c];
@@ -591,48 +588,57 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             }
             if (sliced_tile) {
                 if constexpr (kSliced) {
-                    // ---- the whole tile in the bit-plane domain: lane L owns blocks L and 64 + L
+                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a time.
+                    //      A half tile of blocks with at most kSlicedMaxF planes is at most 64 x 32
+                    //      bytes: three 1 KiB pieces per stream with the alignment shift.  The second
+                    //      half is requested as soon as the first has gone from the registers to LDS.
                     uint8_t *st = s_in[wave];
-                    SlicedIn A[2];
-                    uint32_t shift_c[2];
-                    u32x4 piece[2][kInStageTile / 1024 + 1];
-#pragma unroll
-                    for (int c = 0; c < 2; ++c) {
-                        const uint32_t total = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][kSub]);
+                    constexpr int kPieces = 3;
+                    static_assert(64 * (4 + 4 + 4 * (int)kSlicedMaxF) + 15 <= kPieces * 1024 && kPieces * 1024 <= kInStageTile - 64,
+                                  "a half tile fits its pieces, and the words read beyond its last block the stage");
+                    uint32_t shift_h[2], rel0_h[2];
+                    u32x4 piece[2][kPieces];
+                    auto request_half = [&](int c, int half) __attribute__((always_inline)) {
+                        // blocks 64 half .. 64 half + 63 are sub-steps 4 half .. 4 half + 3
+                        const uint32_t rel0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][4 * half]);
+                        const uint32_t rel1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][4 * half + 4]);
                         const uint32_t room = buf ? room_ctx1[c] : room_ctx0[c];
                         const uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
-                        const uint32_t end = total < lim ? total : lim;
-                        const uintptr_t g0 = (uintptr_t)p.in[c] + (buf ? start_ctx1[c] : start_ctx0[c]);
+                        const uint32_t end = rel1 < lim ? rel1 : lim;
+                        const uintptr_t g0 = (uintptr_t)p.in[c] + (buf ? start_ctx1[c] : start_ctx0[c]) + rel0;
                         const uintptr_t ga = g0 & ~(uintptr_t)15;
-                        shift_c[c] = (uint32_t)(g0 - ga);
-                        const uint32_t nbytes = end ? shift_c[c] + end : 0u;
+                        shift_h[c] = (uint32_t)(g0 - ga);
+                        rel0_h[c] = rel0;
+                        const uint32_t nbytes = end > rel0 ? shift_h[c] + (end - rel0) : 0u;
                         const __amdgpu_buffer_rsrc_t rs = buffer_of(reinterpret_cast<const void *>(ga), (nbytes + 15u) & ~15u);
 #pragma unroll
-                        for (int i = 0; i < kInStageTile / 1024 + 1; ++i)
-                            piece[c][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (lane + 64 * i) * 16, 0, kBufCached);
-                    }
-                    SlicedOut out;
+                        for (int i = 0; i < kPieces; ++i)
+                            piece[c][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 1024 * i, kBufCached);
+                    };
                     auto stage_stream = [&](int c) __attribute__((always_inline)) {
 #pragma unroll
-                        for (int i = 0; i < kInStageTile / 1024 + 1; ++i)
-                            if ((lane + 64 * i) * 16 < kInStageTile)
-                                *reinterpret_cast<u32x4 *>(st + (lane + 64 * i) * 16) = piece[c][i];
+                        for (int i = 0; i < kPieces; ++i) *reinterpret_cast<u32x4 *>(st + (lane + 64 * i) * 16) = piece[c][i];
                         wave_lds_fence();
                     };
                     auto read_block = [&](int c, int half, SlicedIn &blk) __attribute__((always_inline)) {
                         const int b = half * 64 + lane;
-                        sliced_read(st, shift_c[c] + s_ofs_in[wave][c][buf][b], s_hdr_in[wave][c][buf][b], blk);
+                        sliced_read(st, shift_h[c] + s_ofs_in[wave][c][buf][b] - rel0_h[c], s_hdr_in[wave][c][buf][b], blk);
                     };
-                    stage_stream(0);
-                    read_block(0, 0, A[0]);
-                    read_block(0, 1, A[1]);
-                    wave_lds_fence();
-                    stage_stream(1);
+                    request_half(0, 0);
+                    request_half(1, 0);
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
-                        SlicedIn B;
+                        SlicedIn A, B;
+                        SlicedOut out;
+                        stage_stream(0);
+                        read_block(0, half, A);
+                        wave_lds_fence();
+                        if (half == 0) request_half(0, 1);   // after read_block: it replaces shift_h / rel0_h of the stream
+                        stage_stream(1);
                         read_block(1, half, B);
-                        sliced_add(A[half], B, out);
+                        wave_lds_fence();
+                        if (half == 0) request_half(1, 1);
+                        sliced_add(A, B, out);
                         s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
                         const uint32_t incl = wave_incl_scan_u32(out.size, lane);
                         const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
