@@ -582,8 +582,8 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             };
             bool sliced_tile = false;
             if constexpr (kSliced) {
-                // 32 blocks of at most 40 bytes must fit an empty slot (they are written at once)
-                sliced_tile = p.sliced && slot_cap >= 32u * 40u + 16u &&
+                // 32 blocks (outlier bytes, sign word, kSlicedOutPlanes planes) must fit an empty slot: they are written at once
+                sliced_tile = p.sliced && slot_cap >= 32u * (8u + 4u * (uint32_t)kSlicedOutPlanes) + 16u &&
                               (buf ? few_ctx1[0] && few_ctx1[1] : few_ctx0[0] && few_ctx0[1]);
             }
             if (sliced_tile) {
