@@ -112,17 +112,17 @@ int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::Til
 
 // LDS stage per data wave (two deferred tiles by default), in three budgets that let 4, 3 and 2
 // workgroups share a compute unit (with the LDS the kernels hold besides: 0.6 KiB for compress,
-// 12.5 KiB with one incoming stream, 21.1 KiB with two).  The slots hold tiles of streams
+// 12.5 KiB with one incoming stream, 19.4 KiB with two).  The slots hold tiles of streams
 // compressed about 4.6x / 2.9x / 2x or better for compress, 6x / 3.7x / 2x for the sums with one
-// incoming stream and 9x / 4.8x / 2.6x with two.  A tile beyond its slot still works (it goes
+// incoming stream and 9x / 4.5x / 2.5x with two.  A tile beyond its slot still works (it goes
 // through the spill area), so the choice below is a performance heuristic, never a correctness
 // matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
-// fits a compute unit, which is slower than spilling: its largest slots are 7 KiB.)
+// fits a compute unit, which is slower than spilling: its largest slots are 7.3 KiB.)
 constexpr int kStageClasses = 3;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
-    {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (3888 + 64)},
-    {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7216 + 64)}};
+    {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4112 + 64)},
+    {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7440 + 64)}};
 
 // The stream-producing kernels of this process never overlap on a device.  Each of them needs
 // its whole grid resident (the scan's waits), and two such grids from different streams can each

@@ -244,7 +244,7 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
 constexpr int kSub = kTileBlocks / 16;
 constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
 // stream (+) stream stages whole tiles of few planes for the sums in the bit-plane domain
-constexpr int kInStageTile = 3584;   // half a tile of such blocks (three 1 KiB pieces) and the words read beyond its last block
+constexpr int kInStageTile = 3 * 1024 + 64;   // half a tile of such blocks (three 1 KiB pieces) and the words read beyond its last block
 
 template <int LOCAL>
 struct SubRegs {
