@@ -448,6 +448,7 @@ struct SlicedIn {
 
 // The lane's block of an incoming stream from the LDS stage (`p0` = the block's first byte);
 // digest 0 (no payload, or not to be read) gives a block of zeros.
+template <uint32_t NP>   // planes that any block of the wave can have (the others are left zero without being read)
 __device__ __forceinline__ void sliced_read(const uint8_t *stage, uint32_t p0, uint32_t digest, SlicedIn &b)
 {
     const uint32_t F = digest & 0x1fu;
@@ -458,7 +459,9 @@ __device__ __forceinline__ void sliced_read(const uint8_t *stage, uint32_t p0, u
     const uint32_t sign = load_u32_any(stage + p0 + b.ob);
     b.sign = digest ? sign : 0u;
 #pragma unroll
-    for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+    for (uint32_t q = 0; q < kSlicedMaxF; ++q) b.pl[q] = 0u;
+#pragma unroll
+    for (uint32_t q = 0; q < NP; ++q) {
         const uint32_t w = load_u32_any(stage + p0 + b.ob + 4u + 4u * q);
         b.pl[q] = q < F ? w : 0u;
     }
@@ -470,6 +473,7 @@ struct SlicedOut {
 
 // delta_out = delta_A + delta_B for the lane's block, and the block's rate selection
 // (HomComp/src/GSZ.cu:151-167).
+template <uint32_t NP>   // planes that any of the wave's blocks of either stream can have; the sums have NP + 1
 __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B, SlicedOut &o)
 {
     constexpr uint32_t E = 0x80u;   // element 0
@@ -478,7 +482,7 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
     {
         uint32_t anyA = 0, anyB = 0;
 #pragma unroll
-        for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+        for (uint32_t q = 0; q < NP; ++q) {
             anyA |= A.pl[q];
             anyB |= B.pl[q];
         }
@@ -486,7 +490,7 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
         if (__builtin_amdgcn_ballot_w64(gatherA || gatherB) != 0) {   // wave-uniform; rare where outlier mode prevails
             uint32_t gA = 0, gB = 0;
 #pragma unroll
-            for (uint32_t q = 0; q < kSlicedMaxF; ++q) {
+            for (uint32_t q = 0; q < NP; ++q) {
                 gA |= ((A.pl[q] >> 7) & 1u) << q;
                 gB |= ((B.pl[q] >> 7) & 1u) << q;
             }
@@ -500,23 +504,23 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
     o.a0 = (uint32_t)((int32_t)s0 > s0neg ? (int32_t)s0 : s0neg);   // |s0| (0x80000000 stays)
     // ---- elements 1..31, plane by plane
     const uint32_t SA = A.sign & ~E, SB = B.sign & ~E;
-    uint32_t cA = SA, cB = SB, carry = 0, r[kSlicedMaxF + 2];
+    uint32_t cA = SA, cB = SB, carry = 0, r[NP + 2];
 #pragma unroll
-    for (uint32_t q = 0; q < kSlicedMaxF + 2; ++q) {
-        const uint32_t tA = (q < kSlicedMaxF ? A.pl[q] & ~E : 0u) ^ SA;
-        const uint32_t tB = (q < kSlicedMaxF ? B.pl[q] & ~E : 0u) ^ SB;
+    for (uint32_t q = 0; q < NP + 2; ++q) {
+        const uint32_t tA = (q < NP ? A.pl[q] & ~E : 0u) ^ SA;
+        const uint32_t tB = (q < NP ? B.pl[q] & ~E : 0u) ^ SB;
         const uint32_t xA = tA ^ cA, xB = tB ^ cB;
         cA &= tA;
         cB &= tB;
         r[q] = xA ^ xB ^ carry;
         carry = (xA & xB) | (carry & (xA ^ xB));
     }
-    const uint32_t SR = r[kSlicedMaxF + 1];   // the sign plane: the sums fit kSlicedMaxF + 1 bits
+    const uint32_t SR = r[NP + 1];   // the sign plane: the sums fit NP + 1 bits
     uint32_t c = SR, nz = 0;
 #pragma unroll
     for (uint32_t q = 0; q < kSlicedOutPlanes; ++q) o.m[q] = 0;
 #pragma unroll
-    for (uint32_t q = 0; q < kSlicedMaxF + 1; ++q) {
+    for (uint32_t q = 0; q < NP + 1; ++q) {
         const uint32_t t = r[q] ^ SR;
         o.m[q] = t ^ c;
         c &= t;
@@ -540,19 +544,20 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
     const uint32_t ins = plain ? o.a0 : 0u;
     if (__builtin_amdgcn_ballot_w64(ins != 0u) != 0) {
 #pragma unroll
-        for (uint32_t q = 0; q < kSlicedOutPlanes; ++q) o.m[q] |= ((ins >> q) & 1u) << 7;
+        for (uint32_t q = 0; q < NP + 2; ++q) o.m[q] |= ((ins >> q) & 1u) << 7;
     }
 }
 
 // The block's payload at `pos` of the stage: outlier bytes (a whole word is stored; what it
 // writes beyond them is overwritten by the sign word), sign word, planes.
+template <uint32_t NP>
 __device__ __forceinline__ void sliced_write(lds_bytes stage, uint32_t pos, const SlicedOut &o)
 {
     if (o.hdr == 0u) return;
     if (o.ob) store_u32_any(stage + pos, o.a0);
     store_u32_any(stage + pos + o.ob, o.sign);
 #pragma unroll
-    for (uint32_t q = 0; q < (uint32_t)kSlicedOutPlanes; ++q)
+    for (uint32_t q = 0; q < NP + 2; ++q)
         if (q < o.F) store_u32_any(stage + pos + o.ob + 4u + 4u * q, o.m[q]);
 }
 

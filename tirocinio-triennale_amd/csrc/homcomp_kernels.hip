@@ -620,9 +620,19 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         for (int i = 0; i < kPieces; ++i) *reinterpret_cast<u32x4 *>(st + (lane + 64 * i) * 16) = piece[c][i];
                         wave_lds_fence();
                     };
-                    auto read_block = [&](int c, int half, SlicedIn &blk) __attribute__((always_inline)) {
+                    // Most streams this path sees have one to three planes per block: a wave none of
+                    // whose blocks (of the half, either stream) has more takes the code for three.
+                    constexpr uint32_t kFewer = 3;
+                    auto read_block = [&](int c, int half, SlicedIn &blk, bool &fewer) __attribute__((always_inline)) {
                         const int b = half * 64 + lane;
-                        sliced_read(st, shift_h[c] + s_ofs_in[wave][c][buf][b] - rel0_h[c], s_hdr_in[wave][c][buf][b], blk);
+                        const uint32_t digest = s_hdr_in[wave][c][buf][b];
+                        const uint32_t p0 = shift_h[c] + s_ofs_in[wave][c][buf][b] - rel0_h[c];
+                        if (__builtin_amdgcn_ballot_w64((digest & 0x1fu) > kFewer) == 0) {
+                            sliced_read<kFewer>(st, p0, digest, blk);
+                        } else {
+                            sliced_read<kSlicedMaxF>(st, p0, digest, blk);
+                            fewer = false;
+                        }
                     };
                     request_half(0, 0);
                     request_half(1, 0);
@@ -630,15 +640,19 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     for (int half = 0; half < 2; ++half) {
                         SlicedIn A, B;
                         SlicedOut out;
+                        bool fewer = true;
                         stage_stream(0);
-                        read_block(0, half, A);
+                        read_block(0, half, A, fewer);
                         wave_lds_fence();
                         if (half == 0) request_half(0, 1);   // after read_block: it replaces shift_h / rel0_h of the stream
                         stage_stream(1);
-                        read_block(1, half, B);
+                        read_block(1, half, B, fewer);
                         wave_lds_fence();
                         if (half == 0) request_half(1, 1);
-                        sliced_add(A, B, out);
+                        if (fewer)
+                            sliced_add<kFewer>(A, B, out);
+                        else
+                            sliced_add<kSlicedMaxF>(A, B, out);
                         s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
                         const uint32_t incl = wave_incl_scan_u32(out.size, lane);
                         const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
@@ -649,7 +663,12 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                             const uint32_t bytes = q ? all64 - first32 : first32;
                             make_room(bytes);   // always true here: 32 blocks fit an empty slot
                             const uint32_t pos = run - flushed + (incl - out.size) - (q ? first32 : 0u);
-                            if ((lane >> 5) == q) sliced_write((lds_bytes)stage, pos, out);
+                            if ((lane >> 5) == q) {
+                                if (fewer)
+                                    sliced_write<kFewer>((lds_bytes)stage, pos, out);
+                                else
+                                    sliced_write<kSlicedMaxF>((lds_bytes)stage, pos, out);
+                            }
                             run += bytes;
                         }
                     }
