@@ -383,7 +383,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // bytes of the stream from the tile's payload start to its stated end, saturated to 32 bits:
     // everything inside a tile is 32-bit arithmetic against these
     uint32_t room_ctx0[kIn], room_ctx1[kIn];
-    bool few_ctx0[kIn], few_ctx1[kIn];   // kSliced: no block of the tile has more than kSlicedMaxF planes
+    uint32_t few_ctx = 0;   // kSliced: bit b set = no block of the tile in context b (either stream) has more than kSlicedMaxF planes
     auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             int64_t t = tile_of(r);
@@ -419,18 +419,18 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     const uint32_t d0 = z0 != 0u && o0 < room ? header_digest(h0) : 0u;
                     const uint32_t d1 = z1 != 0u && o1 < room ? header_digest(h1) : 0u;
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
-                    bool few = false;
                     if constexpr (kSliced) {
-                        few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0;
+                        const bool few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0;
+                        const uint32_t bit = 1u << b;
+                        if (c == 0) few_ctx |= bit;
+                        if (!few) few_ctx &= ~bit;
                     }
                     if (b) {
                         start_ctx1[c] = start_next[c];
                         room_ctx1[c] = room;
-                        few_ctx1[c] = few;
                     } else {
                         start_ctx0[c] = start_next[c];
                         room_ctx0[c] = room;
-                        few_ctx0[c] = few;
                     }
                 }
                 wave_lds_fence();
@@ -584,7 +584,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
             if constexpr (kSliced) {
                 // 32 blocks (outlier bytes, sign word, kSlicedOutPlanes planes) must fit an empty slot: they are written at once
                 sliced_tile = p.sliced && slot_cap >= 32u * (8u + 4u * (uint32_t)kSlicedOutPlanes) + 16u &&
-                              (buf ? few_ctx1[0] && few_ctx1[1] : few_ctx0[0] && few_ctx0[1]);
+                              ((few_ctx >> buf) & 1u);
             }
             if (sliced_tile) {
                 if constexpr (kSliced) {
