@@ -23,6 +23,15 @@
  *     gives that number.
  *   - A workspace holds the scan state of one call at a time: calls sharing a workspace must be
  *     ordered on one stream (or otherwise serialised).  Use one workspace per concurrent stream.
+ *   - An INPUT stream buffer must be readable up to cmp_size + 160 bytes (or up to
+ *     homcomp_max_stream_bytes(nbEle), whichever is smaller): a block whose payload starts below
+ *     the stated size is fetched in full (the out-of-bound rule of src/GSZ.cu:908-911 looks at the
+ *     block's start only), in whole 16-byte pieces.  Buffers of homcomp_max_stream_bytes always do.
+ *   - Stream-producing kernels keep their whole grid resident and wait for each other's scan
+ *     words, so the library orders such launches of one process on a device, also across
+ *     streams.  Launches recorded into a HIP graph are outside that order: a replay must not
+ *     run at the same time as another stream-producing call or replay on the device (order them
+ *     on one stream or with events), and must end before its workspace is destroyed.
  *   - Every function returns HOMCOMP_OK (0) or a negative HOMCOMP_ERR_* code; no call aborts.
  */
 #ifndef HOMCOMP_H
@@ -41,8 +50,10 @@ extern "C" {
 #define HOMCOMP_ERR_TOO_LARGE (-3)    /* nbEle exceeds the workspace's max_nbEle                */
 #define HOMCOMP_ERR_HIP (-4)          /* a HIP runtime call failed; see homcomp_last_hip_error  */
 #define HOMCOMP_ERR_NO_DEVICE (-5)    /* no usable GPU                                           */
-#define HOMCOMP_ERR_SCAN_TIMEOUT (-6) /* a kernel gave up waiting in the offset scan (sticky);   */
-                                      /* streams produced since workspace creation are invalid   */
+#define HOMCOMP_ERR_SCAN_TIMEOUT (-6) /* a kernel gave up waiting in the offset scan; reported    */
+                                      /* by homcomp_last_size, which also clears it: the streams */
+                                      /* produced on the workspace since the previous            */
+                                      /* homcomp_last_size are invalid, later calls are not      */
 
 typedef struct homcomp_workspace homcomp_workspace;
 
@@ -63,6 +74,18 @@ size_t homcomp_ref_cmpsize(size_t stream_len, size_t nbEle);
  * allreduce_ring_comprs_hom_sum_F_opt hoists out of its loop (src/cuda_awareallreduce.cu:745-760). */
 int homcomp_workspace_create(homcomp_workspace **ws, size_t max_nbEle);
 int homcomp_workspace_destroy(homcomp_workspace *ws);
+/* Tuning of a workspace; no counterpart in the reference, whose one-warp thread blocks wait for
+ * their predecessors without a bound (src/GSZ.cu:196-223).
+ *   HOMCOMP_OPT_GRID_PERCENT  share of the device a stream-producing launch of ws occupies, 1..100
+ *       percent of the resident grid (default 100, or the environment variable
+ *       HOMCOMP_GRID_PERCENT at creation).  The launch needs all its workgroups resident at once;
+ *       where other kernels hold compute units for longer than the bounded waits (tens of
+ *       milliseconds) a full grid ends in HOMCOMP_ERR_SCAN_TIMEOUT, a smaller one fits beside them.
+ *   HOMCOMP_OPT_SPIN_LIMIT    unsuccessful re-reads of a scan word before a wave gives up, 0..2^30
+ *       (default 65536, or HOMCOMP_SPIN_LIMIT at creation). */
+#define HOMCOMP_OPT_GRID_PERCENT 1
+#define HOMCOMP_OPT_SPIN_LIMIT 2
+int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value);
 
 /* GSZ_compress_deviceptr_outlier (include/GSZ_entry.h:14-16, src/GSZ_entry.cu:263-301).
  * d_stream_len (optional, device uint64) receives L when the kernel finishes. */
@@ -106,8 +129,10 @@ int homcomp_range_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, 
 float homcomp_rel_to_abs(float rel, float vmin, float vmax);
 
 /* The blocking read-back of src/GSZ_entry.cu:291 (cudaMemcpy of cmpOffset[gsize-1]): waits for
- * `stream` and returns the length L produced by the last stream-producing call on ws.  Also
- * reports HOMCOMP_ERR_SCAN_TIMEOUT if any kernel on ws had to abandon its bounded wait. */
+ * `stream` and returns the length L produced by the last stream-producing call on ws.  Returns
+ * HOMCOMP_ERR_SCAN_TIMEOUT if a kernel on ws had to abandon its bounded wait since the previous
+ * homcomp_last_size (the output of those calls is incomplete, nothing was written outside the
+ * output buffers) and clears that state, so the calls can be repeated on the same workspace. */
 int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream);
 
 #ifdef __cplusplus

@@ -225,7 +225,9 @@ def test_integer_homomorphism(orc, gen, n):
     assert np.array_equal(h, want)
     # stream (+) stream and the int-delta variant agree with the fused one
     assert np.array_equal(orc.hom_add(sa, orc.compress(b, eb), n), h)
-    assert np.array_equal(orc.hom_sum_i32(sa, orc.quant_predict(b, eb, padded=True)[:npad]), h) or n % 32
+    # (padded=True continues the deltas over the zero padding as the float path sees it: the first
+    # padded delta is -q[n-1], so the ragged length gives the same bytes too)
+    assert np.array_equal(orc.hom_sum_i32(sa, orc.quant_predict(b, eb, padded=True)[:npad]), h)
     # three-way sum is independent of the order (integer addition commutes)
     h1 = orc.hom_sum_f32(orc.hom_sum_f32(sa, b, eb), c, eb)
     h2 = orc.hom_sum_f32(orc.hom_sum_f32(orc.compress(c, eb), a, eb), b, eb)

@@ -18,10 +18,15 @@ LIB_PATH = os.path.join(_HERE, "libhomcomp_amd.so")
 EXPORTS = (
     "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
     "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
-    "homcomp_workspace_destroy", "homcomp_compress_f32", "homcomp_decompress_f32",
+    "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_compress_f32", "homcomp_decompress_f32",
     "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add",
     "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
 )
+
+
+OPT_GRID_PERCENT = 1
+OPT_SPIN_LIMIT = 2
+ERR_SCAN_TIMEOUT = -6
 
 
 class HomCompError(RuntimeError):
@@ -58,6 +63,7 @@ def lib() -> C.CDLL:
         L.homcomp_ref_cmpsize.restype = sz
         L.homcomp_workspace_create.argtypes = [C.POINTER(vp), sz]
         L.homcomp_workspace_destroy.argtypes = [vp]
+        L.homcomp_workspace_set_option.argtypes = [vp, C.c_int, C.c_long]
         L.homcomp_compress_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_decompress_f32.argtypes = [vp, vp, sz, sz, C.c_float, vp, vp]
         L.homcomp_hom_sum_f32.argtypes = [vp, vp, sz, vp, sz, C.c_float, vp, u64p, vp]
@@ -119,6 +125,9 @@ class Workspace:
         if self._h:
             _check(lib().homcomp_workspace_destroy(self._h), "workspace_destroy")
             self._h = C.c_void_p()
+
+    def set_option(self, option: int, value: int) -> None:
+        _check(lib().homcomp_workspace_set_option(self._h, int(option), int(value)), "workspace_set_option")
 
     def __del__(self):
         try:

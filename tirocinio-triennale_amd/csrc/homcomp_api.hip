@@ -9,6 +9,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "homcomp_kernels.hpp"
 
@@ -16,7 +17,11 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 
-constexpr uint32_t kMaxEpoch = (1u << 22) - 1;
+// Epochs 1 .. kMaxEpoch go to eager launches in turn; kGraphEpoch is kept for launches recorded
+// into a graph, which are replayed with the epoch they were captured with and clear the scan
+// words first: an eager call is never handed the epoch whose words a replay left behind.
+constexpr uint32_t kGraphEpoch = (1u << 22) - 1;
+constexpr uint32_t kMaxEpoch = kGraphEpoch - 1;
 // Unsuccessful scan re-reads before a wave gives up (each costs a memory round trip, so this is
 // some tens of milliseconds): long enough for any delay of a resident workgroup, short enough
 // that a launch which could not become resident ends with an error instead of stalling for minutes.
@@ -52,11 +57,12 @@ struct homcomp_workspace {
     float *d_partial;         // min/max partials
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
-    uint32_t max_grid[hc::kOpCount][3];  // resident workgroups of each operation's kernel, per LDS budget (small, medium, large)
+    uint32_t max_grid[hc::kOpCount][3];  // persistent grid of each operation's kernel, per LDS budget (small, medium, large)
+    uint32_t full_grid[hc::kOpCount][3]; // the same at 100 percent (HOMCOMP_OPT_GRID_PERCENT scales it)
     uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
-    uint8_t *d_spill;         // spill slots: four worst-case tiles per data wave
-    uint32_t out_slots;       // deferral depth of packed tiles (2..4)
+    uint32_t out_slots;       // deferral depth of packed tiles (2..4); the device's spill area has this many slots per data wave
+    bool holds_spill;         // counted among the users of the device's spill area
     uint32_t sliced;          // HOMCOMP_SLICED=0 switches the bit-plane path of stream (+) stream off
     int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
 };
@@ -124,36 +130,84 @@ constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4112 + 64)},
     {2 * (8192 + 64), 0, 2 * (8192 + 64), 2 * (8192 + 64), 2 * (7440 + 64)}};
 
-// The stream-producing kernels of this process never overlap on a device.  Each of them needs
-// its whole grid resident (the scan's waits), and two such grids from different streams can each
-// end up half resident, every wave waiting for workgroups that cannot start: both calls would
-// run into the bound of their waits.  So a launch on another stream than the device's previous
-// one first waits (on the GPU, not on the host) for an event recorded on that stream.  A stream
-// under capture is left alone: its graph orders the launches it contains.
-struct DeviceChain {
+// Per-device state shared by all workspaces of the process.
+//
+// Launch chain.  The stream-producing kernels of this process never overlap on a device.  Each of
+// them needs its whole grid resident (the scan's waits), and two such grids from different
+// streams can each end up half resident, every wave waiting for workgroups that cannot start:
+// both calls would run into the bound of their waits.  So a launch on another stream than the
+// device's previous one first waits (on the GPU, not on the host) for an event recorded on that
+// stream.  A stream under capture is left alone: its graph orders the launches it contains.
+//
+// Spill area.  A tile that outgrows its LDS slot waits for its stream offset in global memory:
+// one slot of a worst-case tile per deferred tile and data wave.  Because the kernels that use it
+// never overlap, one area per device serves every workspace; it is allocated with the first
+// workspace, grows to the largest grid x deferral depth asked for, and is freed with the last
+// workspace.  An area that has been outgrown stays allocated until then (a recorded graph may
+// still name it).
+struct DeviceState {
     std::mutex mu;
     hipEvent_t done = nullptr;
     hipStream_t last = nullptr;
     bool any = false;
+    uint8_t *spill = nullptr;
+    size_t spill_bytes = 0;
+    int spill_users = 0;
+    std::vector<void *> retired;
 };
-DeviceChain g_chain[64];
+constexpr int kMaxDevices = 64;
+DeviceState g_dev[kMaxDevices];
 
-int chained_launch(homcomp_workspace *ws, int op, const hc::TileParams &p, uint32_t max_grid, hipStream_t s)
+int spill_acquire(homcomp_workspace *ws, size_t bytes)
+{
+    DeviceState &d = g_dev[ws->device];
+    std::lock_guard<std::mutex> lock(d.mu);
+    if (bytes > d.spill_bytes) {
+        void *area = nullptr;
+        if (!hip_ok(hipMalloc(&area, bytes))) return HOMCOMP_ERR_HIP;
+        if (d.spill) d.retired.push_back(d.spill);
+        d.spill = (uint8_t *)area;
+        d.spill_bytes = bytes;
+    }
+    ++d.spill_users;
+    ws->holds_spill = true;
+    return HOMCOMP_OK;
+}
+
+// after the device has been synchronised
+int spill_release(homcomp_workspace *ws)
+{
+    if (!ws->holds_spill) return HOMCOMP_OK;
+    DeviceState &d = g_dev[ws->device];
+    std::lock_guard<std::mutex> lock(d.mu);
+    ws->holds_spill = false;
+    if (--d.spill_users > 0) return HOMCOMP_OK;
+    int rc = HOMCOMP_OK;
+    if (d.spill && !hip_ok(hipFree(d.spill))) rc = HOMCOMP_ERR_HIP;
+    for (void *area : d.retired)
+        if (!hip_ok(hipFree(area))) rc = HOMCOMP_ERR_HIP;
+    d.retired.clear();
+    d.spill = nullptr;
+    d.spill_bytes = 0;
+    return rc;
+}
+
+int chained_launch(homcomp_workspace *ws, int op, hc::TileParams p, uint32_t max_grid, hipStream_t s)
 {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
-    if (capturing || ws->device < 0 || ws->device >= 64) {
-        if (capturing) {
-            (void)hipGetLastError();
-            // A captured launch is replayed with the epoch it was captured with, so the scan words
-            // of the previous replay would read as this call's: the graph clears them first (with
-            // a kernel; memset nodes are avoided in graphs).
-            if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s))) return HOMCOMP_ERR_HIP;
-        }
+    DeviceState &c = g_dev[ws->device];
+    std::lock_guard<std::mutex> lock(c.mu);
+    p.spill = c.spill;
+    if (capturing) {
+        (void)hipGetLastError();
+        // A captured launch is replayed with the epoch it was captured with, so the scan words
+        // of the previous replay would read as this call's: the graph clears them first (with
+        // a kernel; memset nodes are avoided in graphs).
+        p.epoch = kGraphEpoch;
+        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s))) return HOMCOMP_ERR_HIP;
         return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
-    DeviceChain &c = g_chain[ws->device];
-    std::lock_guard<std::mutex> lock(c.mu);
     if (c.any && c.last != s) {
         // The event is recorded only now, on the stream of the previous launch (a call that stays
         // on one stream pays nothing): it covers that launch and whatever followed it there.
@@ -175,7 +229,6 @@ int chained_launch(homcomp_workspace *ws, int op, const hc::TileParams &p, uint3
 // expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
-    p.spill = ws->d_spill;
     p.out_slots = ws->out_slots;
     p.sliced = ws->sliced;
     int cls = kStageClasses - 1;
@@ -280,6 +333,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
+    if (ws->device < 0 || ws->device >= kMaxDevices) {
+        delete ws;
+        return HOMCOMP_ERR_NO_DEVICE;
+    }
     const size_t t = ws->max_tiles;
     size_t off = 0;
     auto take = [&off](size_t bytes) { size_t o = off; off = (off + bytes + 255) & ~(size_t)255; return o; };
@@ -303,23 +360,28 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
             // one compute unit's worth of workgroups is left free: the persistent grid must be fully
             // resident, and an estimate that is off by a single workgroup would stall the launch
             const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
-            uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
-            // HOMCOMP_GRID_PERCENT (1..100) shrinks the persistent grid, for devices that are shared
-            // with other work and cannot keep a full grid of this library resident
-            if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
-                const long pct = std::strtol(e, nullptr, 10);
-                if (pct >= 1 && pct <= 100) g = (uint32_t)((uint64_t)g * (uint64_t)pct / 100u);
-            }
-            if (g < 2) g = 2;   // an encoder needs a data workgroup and the scan server
-            ws->max_grid[op][cls] = g;
+            const uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
+            ws->full_grid[op][cls] = g;
             if (op != hc::kOpDecompress && g > widest) widest = g;
         }
     }
+    ws->out_slots = 2;
+    if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
+        const long v = std::strtol(e, nullptr, 10);
+        if (v >= 2 && v <= 4) ws->out_slots = (uint32_t)v;
+    }
     if (ok) {
-        // four spill slots per data wave of the widest encoder grid, no more waves than tiles
+        // HOMCOMP_GRID_PERCENT (1..100): the initial value of HOMCOMP_OPT_GRID_PERCENT
+        long pct = 100;
+        if (const char *e = std::getenv("HOMCOMP_GRID_PERCENT")) {
+            const long v = std::strtol(e, nullptr, 10);
+            if (v >= 1 && v <= 100) pct = v;
+        }
+        homcomp_workspace_set_option(ws, HOMCOMP_OPT_GRID_PERCENT, pct);
+        // a spill slot per deferred tile and data wave of the widest encoder grid, no more waves than tiles
         size_t waves = (size_t)(widest > 1 ? widest - 1 : 1) * 4;
         if (waves > ws->max_tiles) waves = ws->max_tiles;
-        ok = hip_ok(hipMalloc((void **)&ws->d_spill, waves * 4 * hc::kSpillSlotBytes));
+        ok = spill_acquire(ws, waves * ws->out_slots * hc::kSpillSlotBytes) == HOMCOMP_OK;
     }
     ws->stage_class = -1;
     if (const char *e = std::getenv("HOMCOMP_STAGE")) {
@@ -329,20 +391,20 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     }
     ws->sliced = 1;
     if (const char *e = std::getenv("HOMCOMP_SLICED")) ws->sliced = std::strtol(e, nullptr, 10) != 0;
-    ws->out_slots = 2;
-    if (const char *e = std::getenv("HOMCOMP_SLOTS")) {
-        const long v = std::strtol(e, nullptr, 10);
-        if (v >= 2 && v <= 4) ws->out_slots = (uint32_t)v;
-    }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {
         const long v = std::strtol(e, nullptr, 10);
-        if (v >= 1 && v <= (1l << 30)) ws->spin_limit = (uint32_t)v;
+        if (v >= 0 && v <= (1l << 30)) ws->spin_limit = (uint32_t)v;
+    }
+    // HOMCOMP_EPOCH_START: the epoch handed out last before the first call (tests cross the wrap with it)
+    if (const char *e = std::getenv("HOMCOMP_EPOCH_START")) {
+        const long v = std::strtol(e, nullptr, 10);
+        if (v >= 0 && v <= (long)kMaxEpoch) ws->epoch = (uint32_t)v;
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
         !hip_ok(hipHostMalloc((void **)&ws->h_total, (2 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
-        if (ws->d_spill) (void)hipFree(ws->d_spill);
+        (void)spill_release(ws);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
@@ -362,13 +424,36 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     return HOMCOMP_OK;
 }
 
+int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value)
+{
+    if (!ws) return HOMCOMP_ERR_INVALID_ARG;
+    switch (option) {
+    case HOMCOMP_OPT_GRID_PERCENT:
+        if (value < 1 || value > 100) return HOMCOMP_ERR_INVALID_ARG;
+        for (int op = 0; op < hc::kOpCount; ++op) {
+            for (int cls = 0; cls < kStageClasses; ++cls) {
+                uint32_t g = (uint32_t)((uint64_t)ws->full_grid[op][cls] * (uint64_t)value / 100u);
+                if (g < 2) g = 2;   // an encoder needs a data workgroup and the scan server
+                ws->max_grid[op][cls] = g;
+            }
+        }
+        return HOMCOMP_OK;
+    case HOMCOMP_OPT_SPIN_LIMIT:
+        if (value < 0 || value > (1l << 30)) return HOMCOMP_ERR_INVALID_ARG;
+        ws->spin_limit = (uint32_t)value;
+        return HOMCOMP_OK;
+    default:
+        return HOMCOMP_ERR_INVALID_ARG;
+    }
+}
+
 int homcomp_workspace_destroy(homcomp_workspace *ws)
 {
     if (!ws) return HOMCOMP_OK;
     int rc = HOMCOMP_OK;
     if (!hip_ok(hipDeviceSynchronize())) rc = HOMCOMP_ERR_HIP;
     if (!hip_ok(hipFree(ws->d_block))) rc = HOMCOMP_ERR_HIP;
-    if (ws->d_spill && !hip_ok(hipFree(ws->d_spill))) rc = HOMCOMP_ERR_HIP;
+    if (spill_release(ws) != HOMCOMP_OK) rc = HOMCOMP_ERR_HIP;
     if (!hip_ok(hipHostFree(ws->h_total))) rc = HOMCOMP_ERR_HIP;
     delete ws;
     return rc;
@@ -516,7 +601,10 @@ int homcomp_last_size(homcomp_workspace *ws, size_t *stream_len, void *stream)
         !hip_ok(hipStreamSynchronize(s)))
         return HOMCOMP_ERR_HIP;
     *stream_len = (size_t)ws->h_total[0];
-    return (uint32_t)ws->h_total[1] ? HOMCOMP_ERR_SCAN_TIMEOUT : HOMCOMP_OK;
+    if ((uint32_t)ws->h_total[1] == 0) return HOMCOMP_OK;
+    // reported once: the flag is cleared (on the same stream) so that the workspace can go on
+    if (!hip_ok(hc::launch_fill_u64(ws->d_total + 1, 1, s))) return HOMCOMP_ERR_HIP;
+    return HOMCOMP_ERR_SCAN_TIMEOUT;
 }
 
 }  // extern "C"

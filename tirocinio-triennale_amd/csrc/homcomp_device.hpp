@@ -647,16 +647,21 @@ __device__ __forceinline__ uint64_t scan_probe(const ScanCtx &c, uint32_t tile)
     return status_load(&c.prefixes[tile]);
 }
 
-// Exclusive prefix of `tile` from an earlier scan_probe(tile).
-__device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint64_t w)
+// Exclusive prefix of `tile` from an earlier scan_probe(tile).  `ok` is false when the wait ran
+// into its bound: the word read last is not this call's prefix and must not be used as an offset.
+__device__ __forceinline__ uint64_t scan_resolve(const ScanCtx &c, uint32_t tile, uint64_t w, bool &ok)
 {
     uint32_t spins = 0;
+    ok = true;
     // Thousands of waves may wait here at the same time, for words that share a few cache lines
     // with the words the scan server is writing: the pause between two looks keeps them from
     // crowding the server out of those lines (HC_POLL_SLEEP x 64 clocks; between 8 and 128 the
     // time of a 1 GiB call does not depend on it, short calls gain a few percent from short pauses).
     while (status_state(w, c.epoch) != 2u) {
-        if (scan_give_up<HC_POLL_SLEEP>(c, spins)) break;
+        if (scan_give_up<HC_POLL_SLEEP>(c, spins)) {
+            ok = false;
+            break;
+        }
         w = scan_probe(c, tile);
     }
     return w & kValueMask;

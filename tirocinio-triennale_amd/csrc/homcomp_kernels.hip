@@ -145,7 +145,10 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
         uint32_t v[PER], mine = 0;
 #pragma unroll
         for (uint32_t j = 0; j < PER; ++j) {
-            v[j] = in ? (uint32_t)(w[j] & 0xffffffffu) : 0u;   // a tile total is below 2^15
+            // a tile total is at most kTileBlocks * kOutBlockBytes; the cap keeps every prefix within
+            // the caller's buffer even when a wait gave up and a word of an earlier call is summed
+            const uint32_t t = (uint32_t)(w[j] & 0xffffffffu);
+            v[j] = in ? (t < (uint32_t)(kTileBlocks * kOutBlockBytes) ? t : (uint32_t)(kTileBlocks * kOutBlockBytes)) : 0u;
             mine += v[j];
         }
         const uint32_t incl = wave_incl_scan_u32(mine, lane);
@@ -511,7 +514,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         const int buf = (int)(r & 1);
         const int obuf = (int)(r % D);
         uint8_t *stage = s_dyn + (uint32_t)wave * p.stage_bytes + (uint32_t)obuf * slot_bytes;
-        uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * 4u + (uint64_t)obuf) * kSpillSlotBytes : nullptr;
+        uint8_t *slot = kEnc ? p.spill + ((uint64_t)wid * (uint64_t)D + (uint64_t)obuf) * kSpillSlotBytes : nullptr;
 
         // ---- the tile packed D rounds ago goes to its place in the stream
         if constexpr (kEnc) {
@@ -534,14 +537,23 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                     else
                         __builtin_amdgcn_s_setprio(0);
                 }
-                if (lane == 0) excl = scan_resolve(scan, (uint32_t)td, probe);
+                bool got = true;
+                if (lane == 0) excl = scan_resolve(scan, (uint32_t)td, probe, got);
                 excl = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(excl >> 32)) << 32) |
                        (uint32_t)__builtin_amdgcn_readfirstlane((int)excl);
+                // A wait that ran into its bound leaves no offset: the tile is dropped (the call
+                // is reported as failed).  An offset is also only taken when the tiles before
+                // this one can add up to it (each emits at most kTileBlocks * kOutBlockBytes
+                // bytes), so nothing is ever written beyond the capacity the caller provides,
+                // whatever the scan words hold after a failed call.
+                const bool usable = __builtin_amdgcn_readfirstlane((int)got) != 0 &&
+                                    excl <= (uint64_t)td * (uint64_t)(kTileBlocks * kOutBlockBytes);
+                if (!usable && lane == 0) atomicOr(scan.err, 1u);
                 uint8_t *dst = p.out_cmp + p.hdr_bytes + excl;
                 // the pieces that went to the spill slot, then what stayed in LDS (behind them in the
                 // slot's numbering: LDS position 0 is the tile's byte `spilled_d`)
-                if (spilled_d) copy_out_spill(slot, dst, spilled_d, lane);
-                if (total_d > spilled_d) copy_out<64>(stage, dst + spilled_d, total_d - spilled_d, lane);
+                if (usable && spilled_d) copy_out_spill(slot, dst, spilled_d, lane);
+                if (usable && total_d > spilled_d) copy_out<64>(stage, dst + spilled_d, total_d - spilled_d, lane);
             }
         }
 

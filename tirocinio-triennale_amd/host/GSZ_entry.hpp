@@ -54,10 +54,20 @@ inline homcomp_workspace *workspace(size_t nbEle)
     return cache.ws;
 }
 
-inline void report_size(homcomp_workspace *ws, int rc, size_t nbEle, size_t *cmpSize, hipStream_t stream)
+// Runs a stream-producing call and reads its size back.  A call that ended in
+// HOMCOMP_ERR_SCAN_TIMEOUT (other kernels held compute units, so its grid was not resident as a
+// whole) is repeated once with half the grid, which the workspace then keeps.
+template <typename Launch>
+inline void run_and_report(homcomp_workspace *ws, Launch launch, size_t nbEle, size_t *cmpSize, hipStream_t stream)
 {
     size_t len = 0;
+    int rc = launch();
     if (rc == HOMCOMP_OK) rc = homcomp_last_size(ws, &len, stream);
+    if (rc == HOMCOMP_ERR_SCAN_TIMEOUT) {
+        homcomp_workspace_set_option(ws, HOMCOMP_OPT_GRID_PERCENT, 50);
+        rc = launch();
+        if (rc == HOMCOMP_OK) rc = homcomp_last_size(ws, &len, stream);
+    }
     last_status() = rc;
 #ifdef HOMCOMP_TRUE_CMPSIZE
     *cmpSize = len;
@@ -76,8 +86,9 @@ inline void GSZ_compress_deviceptr_outlier(float *d_oriData, unsigned char *d_cm
 {
     homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
     if (!ws) return;
-    const int rc = homcomp_compress_f32(ws, d_oriData, nbEle, errorBound, d_cmpBytes, nullptr, stream);
-    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+    homcomp::detail::run_and_report(
+        ws, [&] { return homcomp_compress_f32(ws, d_oriData, nbEle, errorBound, d_cmpBytes, nullptr, stream); }, nbEle,
+        cmpSize, stream);
 }
 
 // HomComp/include/GSZ_entry.h:17-20.  cmpSize may be either convention: blocks are only skipped
@@ -100,9 +111,10 @@ inline void homomorphic_sum(unsigned char *d_cmpBytesIn, int *d_quantPredLoc, un
     (void)errorBound;  // the integer path does not quantise
     homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
     if (!ws) return;
-    const int rc = homcomp_hom_sum_i32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_quantPredLoc, nbEle,
-                                       d_cmpByteOut, nullptr, stream);
-    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+    homcomp::detail::run_and_report(
+        ws,
+        [&] { return homcomp_hom_sum_i32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_quantPredLoc, nbEle, d_cmpByteOut, nullptr, stream); },
+        nbEle, cmpSize, stream);
 }
 
 // HomComp/include/GSZ_entry.h:33-36
@@ -112,9 +124,13 @@ inline void homomorphic_sum_F(unsigned char *d_cmpBytesIn, float *d_localChunk, 
 {
     homcomp_workspace *ws = homcomp::detail::workspace(nbEle);
     if (!ws) return;
-    const int rc = homcomp_hom_sum_f32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_localChunk, nbEle, errorBound,
-                                       d_cmpByteOut, nullptr, stream);
-    homcomp::detail::report_size(ws, rc, nbEle, cmpSize, stream);
+    homcomp::detail::run_and_report(
+        ws,
+        [&] {
+            return homcomp_hom_sum_f32(ws, d_cmpBytesIn, cmpSizeCmpBlock, d_localChunk, nbEle, errorBound, d_cmpByteOut,
+                                       nullptr, stream);
+        },
+        nbEle, cmpSize, stream);
 }
 
 // Callers of the reference launch kernel_quant_prediction<<<grid, 32, 0, stream>>>(...) directly

@@ -164,24 +164,36 @@ struct RingCall {
     bool int_deltas;
     hipStream_t stream;
 
-    // GSZ_compress_deviceptr_outlier + size read-back (blocking, as the reference's wrapper)
+    // A stream-producing call and its size read-back (blocking, as the reference's wrappers).  A
+    // call that ended in HOMCOMP_ERR_SCAN_TIMEOUT (kernels of the transport held compute units,
+    // so its grid was not resident as a whole) is repeated once with half the grid, which the
+    // workspace then keeps.
+    template <typename Launch>
+    int sized(Launch launch, size_t *len) const
+    {
+        int rc = launch();
+        if (rc == HOMCOMP_OK) rc = homcomp_last_size(buf.ws, len, stream);
+        if (rc != HOMCOMP_ERR_SCAN_TIMEOUT) return rc;
+        homcomp_workspace_set_option(buf.ws, HOMCOMP_OPT_GRID_PERCENT, 50);
+        rc = launch();
+        return rc != HOMCOMP_OK ? rc : homcomp_last_size(buf.ws, len, stream);
+    }
+    // GSZ_compress_deviceptr_outlier
     int compress(const float *d_block, size_t n, unsigned char *d_out, size_t *len) const
     {
-        const int rc = homcomp_compress_f32(buf.ws, d_block, n, eb, d_out, nullptr, stream);
-        return rc != HOMCOMP_OK ? rc : homcomp_last_size(buf.ws, len, stream);
+        return sized([&] { return homcomp_compress_f32(buf.ws, d_block, n, eb, d_out, nullptr, stream); }, len);
     }
     // homomorphic_sum_F, or kernel_quant_prediction + homomorphic_sum (:61-72)
     int hom_sum(const unsigned char *d_in, size_t in_len, const float *d_block, size_t n, unsigned char *d_out,
                 size_t *len) const
     {
-        int rc;
         if (int_deltas) {
-            rc = homcomp_quant_predict_f32(d_block, n, eb, buf.d_quant, stream);
-            if (rc == HOMCOMP_OK) rc = homcomp_hom_sum_i32(buf.ws, d_in, in_len, buf.d_quant, n, d_out, nullptr, stream);
-        } else {
-            rc = homcomp_hom_sum_f32(buf.ws, d_in, in_len, d_block, n, eb, d_out, nullptr, stream);
+            const int rc = homcomp_quant_predict_f32(d_block, n, eb, buf.d_quant, stream);
+            if (rc != HOMCOMP_OK) return rc;
+            return sized([&] { return homcomp_hom_sum_i32(buf.ws, d_in, in_len, buf.d_quant, n, d_out, nullptr, stream); },
+                         len);
         }
-        return rc != HOMCOMP_OK ? rc : homcomp_last_size(buf.ws, len, stream);
+        return sized([&] { return homcomp_hom_sum_f32(buf.ws, d_in, in_len, d_block, n, eb, d_out, nullptr, stream); }, len);
     }
     int decompress(const unsigned char *d_in, size_t in_len, float *d_block, size_t n) const
     {
