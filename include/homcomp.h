@@ -117,6 +117,25 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
                     const unsigned char *d_cmp_b, size_t size_b, size_t nbEle,
                     unsigned char *d_cmp_out, uint64_t *d_stream_len, void *stream);
 
+/* homcomp_hom_sum_f32 for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * wrapper allocates, zeroes and frees six arrays per call, src/GSZ_entry.cu:519-548).  No
+ * workspace: the scan words, the incoming stream's tile offsets and the spill area live in one
+ * array of about 28.3 MiB inside the library, which every GPU the library runs on holds until
+ * the process ends.  The call allocates and frees nothing (the first call on a device looks up
+ * the array's address and the kernel's resident grid; make it outside a capture).
+ *   - nbEle is at most HOMCOMP_STATIC_MAX_ELEMENTS, else HOMCOMP_ERR_TOO_LARGE.
+ *   - d_result (required, device uint64[2]): [0] receives the stream length L, [1] is non-zero
+ *     when a wave gave up waiting in the offset scan (the output is then invalid).
+ *   - The array is shared by all calls on a GPU and keeps the last call's contents (the call
+ *     clears what it needs): two calls that overlap on one GPU race, so issue them on one stream
+ *     or order them with events.  Results equal homcomp_hom_sum_f32's byte for byte; the grid is
+ *     capped at 224 data workgroups, so calls beyond about 3.6 M elements run below its speed. */
+#define HOMCOMP_STATIC_MAX_ELEMENTS ((size_t)1 << 24)
+int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size, const float *d_local,
+                               size_t nbEle, float eb, unsigned char *d_cmp_out, uint64_t *d_result,
+                               void *stream);
+
 /* kernel_quant_prediction (include/homcomp.cuh:2-5, src/homcomp.cu:1553-1602), which callers of
  * the reference launch directly.  Writes nbEle int32 deltas. */
 int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,

@@ -19,7 +19,7 @@ EXPORTS = (
     "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
     "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
     "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_compress_f32", "homcomp_decompress_f32",
-    "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add",
+    "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add", "homcomp_hom_sum_f32_static",
     "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
 )
 
@@ -69,6 +69,7 @@ def lib() -> C.CDLL:
         L.homcomp_hom_sum_f32.argtypes = [vp, vp, sz, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_hom_sum_i32.argtypes = [vp, vp, sz, vp, sz, vp, u64p, vp]
         L.homcomp_hom_add.argtypes = [vp, vp, sz, vp, sz, sz, vp, u64p, vp]
+        L.homcomp_hom_sum_f32_static.argtypes = [vp, sz, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_quant_predict_f32.argtypes = [vp, sz, C.c_float, vp, vp]
         L.homcomp_range_f32.argtypes = [vp, vp, sz, vp, vp]
         L.homcomp_rel_to_abs.argtypes = [C.c_float, C.c_float, C.c_float]
@@ -184,6 +185,19 @@ class Workspace:
         out = C.c_size_t()
         _check(lib().homcomp_last_size(self._h, C.byref(out), _stream_ptr(stream)), "last_size")
         return int(out.value)
+
+
+STATIC_MAX_ELEMENTS = 1 << 24
+
+
+def hom_sum_f32_static(cmp_in, cmp_in_size: int, local, eb: float, cmp_out, result, n: int | None = None,
+                       stream=None) -> None:
+    """homcomp_hom_sum_f32_static: no workspace, nothing allocated; ``result`` is a device int64[2]
+    (stream length, scan time-out flag)."""
+    n = local.numel() if n is None else n
+    _check(lib().homcomp_hom_sum_f32_static(cmp_in.data_ptr(), cmp_in_size, local.data_ptr(), n, eb,
+                                            cmp_out.data_ptr(), result.data_ptr(), _stream_ptr(stream)),
+           "hom_sum_f32_static")
 
 
 def quant_predict(data, eb: float, delta, n: int | None = None, stream=None) -> None:

@@ -192,20 +192,23 @@ int spill_release(homcomp_workspace *ws)
     return rc;
 }
 
-int chained_launch(homcomp_workspace *ws, int op, hc::TileParams p, uint32_t max_grid, hipStream_t s)
+// `scan_words` / `n_scan_words`: the scan words of the call, cleared first when the launch is
+// being recorded into a graph.  p.spill == nullptr: the device's spill area is used.
+int chained_launch(int device, uint64_t *scan_words, uint64_t n_scan_words, int op, hc::TileParams p,
+                   uint32_t max_grid, hipStream_t s)
 {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
-    DeviceState &c = g_dev[ws->device];
+    DeviceState &c = g_dev[device];
     std::lock_guard<std::mutex> lock(c.mu);
-    p.spill = c.spill;
+    if (!p.spill) p.spill = c.spill;
     if (capturing) {
         (void)hipGetLastError();
         // A captured launch is replayed with the epoch it was captured with, so the scan words
         // of the previous replay would read as this call's: the graph clears them first (with
         // a kernel; memset nodes are avoided in graphs).
         p.epoch = kGraphEpoch;
-        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s))) return HOMCOMP_ERR_HIP;
+        if (!hip_ok(hc::launch_fill_u64(scan_words, n_scan_words, s))) return HOMCOMP_ERR_HIP;
         return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
     if (c.any && c.last != s) {
@@ -226,40 +229,42 @@ int chained_launch(homcomp_workspace *ws, int op, hc::TileParams p, uint32_t max
     return HOMCOMP_OK;
 }
 
+// LDS budget of a stream-producing call from the payload bytes per tile it is expected to
+// produce (0: unknown, the large budget).
+int choose_stage_class(int op, uint64_t expected_tile_bytes, uint32_t out_slots)
+{
+    if (expected_tile_bytes == 0) return kStageClasses - 1;
+    // the smallest budget whose slots hold the expected tile with an eighth to spare
+    int holds = -1;
+    for (int c = kStageClasses - 1; c >= 0; --c) {
+        const uint64_t slot_cap = kStage[c][op] / out_slots - 64u;
+        if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) holds = c;
+    }
+    // The sums are bound by instruction issue and gain more from a third and fourth
+    // workgroup per compute unit than they lose by spilling, so they never take the large
+    // budget by themselves; compress is bound by memory and avoids the spill traffic
+    // where it can, and where no budget holds the tiles the medium one is its best
+    // balance between waves and spilled bytes.  (Measured on MI355X at 1 GiB, compression
+    // ratios 1.6 to 4.4.)
+    if (op == hc::kOpCompress) return holds < 0 ? 1 : holds;
+    return holds < 0 || holds == kStageClasses - 1 ? 0 : holds;
+}
+
 // expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
     p.out_slots = ws->out_slots;
     p.sliced = ws->sliced;
-    int cls = kStageClasses - 1;
     if (op == hc::kOpDecompress) {
-        cls = 0;
-    } else {
-        if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
-        if (expected_tile_bytes != 0) {
-            // the smallest budget whose slots hold the expected tile with an eighth to spare
-            int holds = -1;
-            for (int c = kStageClasses - 1; c >= 0; --c) {
-                const uint64_t slot_cap = kStage[c][op] / ws->out_slots - 64u;
-                if (expected_tile_bytes + expected_tile_bytes / 8 + 64u <= slot_cap) holds = c;
-            }
-            // The sums are bound by instruction issue and gain more from a third and fourth
-            // workgroup per compute unit than they lose by spilling, so they never take the large
-            // budget by themselves; compress is bound by memory and avoids the spill traffic
-            // where it can, and where no budget holds the tiles the medium one is its best
-            // balance between waves and spilled bytes.  (Measured on MI355X at 1 GiB, compression
-            // ratios 1.6 to 4.4.)
-            if (op == hc::kOpCompress)
-                cls = holds < 0 ? 1 : holds;
-            else
-                cls = holds < 0 || holds == kStageClasses - 1 ? 0 : holds;
-        }
-        if (ws->stage_class >= 0) cls = ws->stage_class;
-        p.host_total = &ws->h_mean_tile[op];
+        p.stage_bytes = 0u;
+        return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
-    p.stage_bytes = op == hc::kOpDecompress ? 0u : kStage[cls][op];
-    if (op == hc::kOpDecompress) return hip_ok(hc::launch_op(op, p, ws->max_grid[op][cls], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
-    return chained_launch(ws, op, p, ws->max_grid[op][cls], s);
+    if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
+    int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
+    if (ws->stage_class >= 0) cls = ws->stage_class;
+    p.host_total = &ws->h_mean_tile[op];
+    p.stage_bytes = kStage[cls][op];
+    return chained_launch(ws->device, ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, op, p, ws->max_grid[op][cls], s);
 }
 
 // payload bytes per tile of an incoming stream
@@ -273,6 +278,73 @@ int empty_stream(homcomp_workspace *ws, uint64_t *d_stream_len, hipStream_t s)
 {
     if (!hip_ok(hc::launch_fill_u64(ws->d_total, 1, s))) return HOMCOMP_ERR_HIP;
     if (d_stream_len && !hip_ok(hc::launch_fill_u64(d_stream_len, 1, s))) return HOMCOMP_ERR_HIP;
+    return HOMCOMP_OK;
+}
+
+// ---------------------------------------------------------------- allocation-free entry point
+//
+// homcomp_hom_sum_f32_static keeps everything a workspace would hold in one device array of the
+// library: scan words, the incoming stream's tile offsets and the scratch of their pre-pass, and
+// a spill area for a grid of kStaticDataGroups data workgroups.  Layout (byte offsets):
+constexpr size_t kStaticMaxElems = HOMCOMP_STATIC_MAX_ELEMENTS;
+constexpr uint32_t kStaticMaxTiles = (uint32_t)(kStaticMaxElems / hc::kHostTileElems);
+constexpr uint32_t kStaticDataGroups = 224;   // data workgroups of four waves
+constexpr uint32_t kStaticSlots = 2;          // deferral depth
+constexpr size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+constexpr size_t kStaticOfsScan = 0;                                                                   // 2 x tiles words
+constexpr size_t kStaticOfsIn = kStaticOfsScan + align256(2 * (size_t)kStaticMaxTiles * 8);            // tiles + 1 offsets
+constexpr size_t kStaticOfsTotals = kStaticOfsIn + align256(((size_t)kStaticMaxTiles + 1) * 8);        // tiles totals
+constexpr size_t kStaticOfsBlocks = kStaticOfsTotals + align256((size_t)kStaticMaxTiles * 4);          // sums over 256 tiles
+constexpr size_t kStaticOfsSpill = kStaticOfsBlocks + align256(((size_t)kStaticMaxTiles / 256 + 1) * 4);
+constexpr size_t kStaticBytes =
+    kStaticOfsSpill + (size_t)kStaticDataGroups * 4 * kStaticSlots * hc::kSpillSlotBytes;   // about 28.3 MiB
+
+}  // namespace
+
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the
+// process ends.  In host code the name is only a handle for hipGetSymbolAddress: the address a
+// kernel can use is looked up once per device (static_state below) and passed as an argument.
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+namespace {
+
+struct StaticState {
+    std::mutex mu;
+    bool ready = false;
+    uint8_t *base = nullptr;                 // device address of `scratch` on this device
+    uint32_t grid[kStageClasses] = {0, 0, 0};  // persistent grid of hom_sum_f32 per LDS budget, scan server included
+};
+StaticState g_static[kMaxDevices];
+
+// First call on a device: the address of the device's copy of `scratch`, the resident grid, and
+// the event of the launch chain, so that later calls create nothing.
+int static_setup(int device, StaticState **out)
+{
+    StaticState &st = g_static[device];
+    std::lock_guard<std::mutex> lock(st.mu);
+    *out = &st;
+    if (st.ready) return HOMCOMP_OK;
+    void *ptr = nullptr;
+    if (!hip_ok(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) || !ptr) return HOMCOMP_ERR_HIP;
+    hipDeviceProp_t prop;
+    if (!hip_ok(hipGetDeviceProperties(&prop, device))) return HOMCOMP_ERR_HIP;
+    for (int cls = 0; cls < kStageClasses; ++cls) {
+        int per_cu = 0;
+        if (!hip_ok(hc::op_kernel_residency(hc::kOpHomSumF32, kStage[cls][hc::kOpHomSumF32], &per_cu))) return HOMCOMP_ERR_HIP;
+        if (per_cu < 1) per_cu = 1;
+        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
+        uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
+        if (g > kStaticDataGroups + 1) g = kStaticDataGroups + 1;   // the spill area holds this many groups
+        if (g < 2) g = 2;
+        st.grid[cls] = g;
+    }
+    {
+        DeviceState &c = g_dev[device];
+        std::lock_guard<std::mutex> chain(c.mu);
+        if (!c.done && !hip_ok(hipEventCreateWithFlags(&c.done, hipEventDisableTiming))) return HOMCOMP_ERR_HIP;
+    }
+    st.base = (uint8_t *)ptr;
+    st.ready = true;
     return HOMCOMP_OK;
 }
 
@@ -566,6 +638,58 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
     if ((rc = in_offsets(ws, 1, d_cmp_b, &p, s))) return rc;
     const uint64_t ta = tile_bytes_of(p, size_a), tb = tile_bytes_of(p, size_b);
     return run_tile_op(ws, hc::kOpHomAdd, p, ta > tb ? ta : tb, s);
+}
+
+int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size, const float *d_local,
+                               size_t nbEle, float eb, unsigned char *d_cmp_out, uint64_t *d_result,
+                               void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    if (!d_result || !eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle > kStaticMaxElems) return HOMCOMP_ERR_TOO_LARGE;
+    // d_result[0] = stream length, d_result[1] = non-zero if a wave gave up waiting in the scan
+    if (!hip_ok(hc::launch_fill_u64(d_result, 2, s))) return HOMCOMP_ERR_HIP;
+    if (nbEle == 0) return HOMCOMP_OK;
+    if (!d_cmp_in || !d_local || !d_cmp_out) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_local)) return HOMCOMP_ERR_ALIGNMENT;
+    int device = -1;
+    if (!hip_ok(hipGetDevice(&device))) return HOMCOMP_ERR_HIP;
+    if (device < 0 || device >= kMaxDevices) return HOMCOMP_ERR_NO_DEVICE;
+    StaticState *st = nullptr;
+    int rc = static_setup(device, &st);
+    if (rc) return rc;
+    uint8_t *base = st->base;
+    hc::TileParams p;
+    std::memset(&p, 0, sizeof p);
+    p.n = nbEle;
+    p.hdr_bytes = homcomp_header_bytes(nbEle);
+    p.n_tiles = (uint32_t)(padded_len(nbEle) / hc::kHostTileElems);
+    p.tile_totals = (uint64_t *)(base + kStaticOfsScan);
+    p.tile_prefixes = p.tile_totals + kStaticMaxTiles;
+    p.spin_limit = kSpinLimit;
+    p.total = d_result;
+    p.error = (uint32_t *)(d_result + 1);
+    p.epoch = 1;   // the scan words of the tiles in use are cleared by every call, so one tag serves
+    p.in[0] = d_cmp_in;
+    p.in_size[0] = cmp_in_size;
+    p.in_ofs[0] = (uint64_t *)(base + kStaticOfsIn);
+    p.local = d_local;
+    p.out_cmp = d_cmp_out;
+    p.eb = eb;
+    p.recip = 0.5f / eb;
+    p.spill = base + kStaticOfsSpill;
+    p.out_slots = kStaticSlots;
+    p.sliced = 1;
+    const int cls = choose_stage_class(hc::kOpHomSumF32, tile_bytes_of(p, cmp_in_size), kStaticSlots);
+    p.stage_bytes = kStage[cls][hc::kOpHomSumF32];
+    // totals and prefixes of the tiles this call uses (the arrays keep the last call's words)
+    if (!hip_ok(hc::launch_fill_u64(p.tile_totals, p.n_tiles, s)) ||
+        !hip_ok(hc::launch_fill_u64(p.tile_prefixes, p.n_tiles, s)))
+        return HOMCOMP_ERR_HIP;
+    if (!hip_ok(hc::launch_in_offsets(d_cmp_in, p.n_tiles, p.hdr_bytes, (uint32_t *)(base + kStaticOfsTotals),
+                                      (uint32_t *)(base + kStaticOfsBlocks), (uint64_t *)(base + kStaticOfsIn), s)))
+        return HOMCOMP_ERR_HIP;
+    return chained_launch(device, nullptr, 0, hc::kOpHomSumF32, p, st->grid[cls], s);
 }
 
 int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,
