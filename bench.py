@@ -24,10 +24,27 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X published peak
 
-# HBM bytes per launch of the dominant kernel (hom_sum_f32) measured with rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE and scaled as described in profiles/pmc_hbm_traffic_smooth_1GiB_rel1e-4.txt;
-# keyed by (kind, log2n, rel).  Other workloads report null.
-MEASURED_TRAFFIC = {("smooth", 28, 1e-4): 1.3437e+09}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(kind: str, log2n: int, rel: float):
+    """HBM bytes per launch of the dominant kernel from the committed counter summary of this
+    workload (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, two runs), with the scaling that summary
+    states; None when no summary of the workload is there."""
+    size = f"{4 * (1 << log2n) // 2**30}GiB" if log2n >= 28 else f"{4 * (1 << log2n) // 2**20}MiB"
+    path = os.path.join(PROFILES, f"pmc_hbm_traffic_{kind}_{size}_rel{rel:g}.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("bench_traffic:"):
+                    kv = dict(item.split("=", 1) for item in line.split()[1:])
+                    return {"bytes": float(kv["bytes"]), "kernel": kv["kernel"],
+                            "calibration": f"FETCH_SIZE x {kv['fetch_scale']} ({kv['fetch_reference']}), "
+                                           f"WRITE_SIZE x {kv['write_scale']} ({kv['write_reference']})",
+                            "source": os.path.relpath(path, ROOT)}
+    except OSError:
+        pass
+    return None
 
 
 def time_op(torch, fn, iters: int) -> float:
@@ -142,6 +159,166 @@ def error_measures(torch, x, y, dec, eb, chunk=1 << 24):
             "correlation": round(cov / math.sqrt(var_o * var_d), 9) if var_o > 0 and var_d > 0 else None}
 
 
+def op_entry(n, ms, alg_bytes):
+    return {"ms": round(ms, 4), "GBps_input": round(4 * n / ms / 1e6, 1),
+            "frac_hbm": round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)}
+
+
+def other_configs(torch, pkg, gen, orc):
+    """The named configurations besides the headline one, each with kernel-side times (HIP events),
+    fraction of the HBM peak (algorithmic bytes), compression ratio and, when the oracle is
+    there, a byte-for-byte comparison of the GPU's streams with the oracle's on the same buffers.
+
+      smooth_64M_rel1e-4 / _rel1e-3   64M smooth values: one compress + one decompress
+      gradient_1GiB_abs1e-6           256M gradient-like values, ABS 1e-6: wide planes, spilled tiles
+      ring_8x32M                      ring reduce-scatter of 8 rank buffers of 32M values in 8 chunks:
+                                      8 compresses + 56 hom_sum_f32 in 7 sequential waves; once with every
+                                      length read back to the host before the next call (what the
+                                      reference's ring does with MPI_Get_count) and once without any
+                                      host round trip (the incoming size is stated as the buffer capacity,
+                                      the lengths stay in device words)
+    """
+    import numpy as np
+    res = {}
+    if orc is not None:
+        orc.set_threads(min(16, os.cpu_count() or 1))
+
+    def same(buf, length, want):
+        return bool(length == want.size and torch.equal(buf[:length], torch.from_numpy(want).cuda()))
+
+    # ---- 64M smooth, REL 1e-4 and 1e-3
+    n = 1 << 26
+    x = gen.smooth_torch(n, seed=1)
+    ws = pkg.Workspace(n)
+    mm = torch.empty(2, dtype=torch.float32, device="cuda")
+    ws.value_range(x, mm)
+    r = mm.cpu().numpy()
+    cap = pkg.max_stream_bytes(n)
+    ca = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    dec = torch.empty(n, dtype=torch.float32, device="cuda")
+    xh = x.cpu().numpy() if orc is not None else None
+    for rel in (1e-4, 1e-3):
+        eb = pkg.rel_to_abs(rel, float(r[0]), float(r[1]))
+        ws.compress(x, eb, ca)
+        la = ws.last_size()
+        e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3),
+             "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10), 4 * n + la),
+             "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(ca, la, n, eb, dec), 10), la + 4 * n)}
+        if orc is not None:
+            want = orc.compress(xh, np.float32(eb))
+            ws.compress(x, eb, ca)
+            ws.last_size()
+            ws.decompress(ca, la, n, eb, dec)
+            torch.cuda.synchronize()
+            wd = orc.decompress(want, n, np.float32(eb))
+            e["matches_oracle"] = same(ca, la, want) and bool(
+                torch.equal(dec.view(torch.int32), torch.from_numpy(wd.view(np.int32)).cuda()))
+        res[f"smooth_64M_rel{rel:g}"] = e
+    del x, ca, dec, ws, xh
+    torch.cuda.empty_cache()
+
+    # ---- 1 GiB gradient-like, ABS 1e-6
+    n = 1 << 28
+    eb = 1e-6
+    x = gen.gradient_like_torch(n, seed=1)
+    y = gen.gradient_like_torch(n, seed=2)
+    ws = pkg.Workspace(n)
+    cap = pkg.max_stream_bytes(n)
+    ca, cb, cs = (torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(3))
+    dec = torch.empty(n, dtype=torch.float32, device="cuda")
+    ws.compress(x, eb, ca)
+    la = ws.last_size()
+    ws.compress(y, eb, cb)
+    lb = ws.last_size()
+    ws.hom_sum_f32(ca, la, y, eb, cs)
+    ls = ws.last_size()
+    e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3), "compression_ratio_sum": round(4 * n / ls, 3),
+         "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 5), 4 * n + la),
+         "hom_sum_f32": op_entry(n, time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), 5), la + 4 * n + ls),
+         "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), 5), ls + 4 * n)}
+    ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8))   # dec doubles as the output buffer: 4N >= L here
+    e["hom_add"] = op_entry(n, time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8)), 5), la + lb + ls)
+    ok = ws.last_size() == ls and bool(torch.equal(dec.view(torch.uint8)[:ls], cs[:ls]))
+    e["hom_add_equals_hom_sum_f32"] = ok
+    if orc is not None:
+        xh, yh = x.cpu().numpy(), y.cpu().numpy()
+        want = orc.compress(xh, np.float32(eb))
+        ok = ok and same(ca, la, want) and same(cs, ls, orc.hom_sum_f32(want, yh, np.float32(eb)))
+        del xh, yh, want
+        e["matches_oracle"] = ok
+    res["gradient_1GiB_abs1e-6"] = e
+    del x, y, ca, cb, cs, dec, ws
+    torch.cuda.empty_cache()
+
+    # ---- ring reduce-scatter, 8 ranks x 32M, 4M-element chunks
+    ranks, n_rank = 8, 1 << 25
+    chunk = n_rank // ranks
+    data = [gen.smooth_torch(n_rank, seed=10 + k) for k in range(ranks)]
+    ws = pkg.Workspace(n_rank)
+    mm = torch.empty(2 * ranks, dtype=torch.float32, device="cuda")
+    for k in range(ranks):
+        ws.value_range(data[k], mm[2 * k:2 * k + 2])
+    m = mm.cpu().numpy()
+    eb = pkg.rel_to_abs(1e-4, float(m[0::2].min()), float(m[1::2].max()))
+    ws.close()
+    ws = pkg.Workspace(chunk)
+    cap = pkg.max_stream_bytes(chunk)
+    cur = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    nxt = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    lens = torch.zeros(ranks, dtype=torch.int64, device="cuda")
+
+    def ring(read_back: bool):
+        a, b = cur, nxt
+        sizes = [cap] * ranks
+        for c in range(ranks):
+            ws.compress(data[c][c * chunk:(c + 1) * chunk], eb, a[c], stream_len=lens[c:c + 1])
+            if read_back:
+                sizes[c] = ws.last_size()
+        for k in range(1, ranks):
+            for c in range(ranks):
+                ws.hom_sum_f32(a[c], sizes[c], data[(c + k) % ranks][c * chunk:(c + 1) * chunk], eb, b[c],
+                               stream_len=lens[c:c + 1])
+                if read_back:
+                    sizes[c] = ws.last_size()
+            a, b = b, a
+        return a
+
+    def timed(read_back: bool):
+        ring(read_back)
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            final = ring(read_back)
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return best * 1e3, final
+
+    ms_dev, final = timed(False)
+    final_lens = [int(v) for v in lens.cpu()]
+    ms_host, final_h = timed(True)
+    e = {"ranks": ranks, "elements_per_rank": n_rank, "chunk_elements": chunk, "eb_abs": eb, "calls": "8 compress + 56 hom_sum_f32",
+         "ms_lengths_on_device": round(ms_dev, 4), "ms_lengths_read_back": round(ms_host, 4),
+         "GBps_rank_data_lengths_on_device": round(ranks * 4 * n_rank / ms_dev / 1e6, 1),
+         "GBps_rank_data_lengths_read_back": round(ranks * 4 * n_rank / ms_host / 1e6, 1),
+         "compression_ratio_reduced": round(ranks * 4 * chunk / sum(final_lens), 3)}
+    ok = all(bool(torch.equal(final[c][:final_lens[c]], final_h[c][:final_lens[c]])) for c in range(ranks))
+    e["both_modes_same_bytes"] = ok
+    if orc is not None:
+        # the oracle's chain for one chunk, and integer addition of the ranks' quantised values for it
+        c = 3
+        host = [d[c * chunk:(c + 1) * chunk].cpu().numpy() for d in data]
+        ref = orc.compress(host[c], np.float32(eb))
+        for k in range(1, ranks):
+            ref = orc.hom_sum_f32(ref, host[(c + k) % ranks], np.float32(eb))
+        q = sum(orc.quantize_array(h, np.float32(eb)).astype(np.int64) for h in host)
+        e["matches_oracle"] = ok and same(final[c], final_lens[c], ref) and bool(
+            np.array_equal(orc.decode_quants(ref, chunk).astype(np.int64), q))
+    res["ring_8x32M"] = e
+    ws.close()
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -154,6 +331,8 @@ def main() -> int:
     ap.add_argument("--cpu-sample-log2", type=int, default=28,
                     help="the CPU baseline runs on the first 2^k elements of each operand (default: the whole workload)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="only the headline workload (profiling runs); default: the other named configurations follow it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1:1 copy of an operand (reference point for HBM counters)")
     ap.add_argument("--sweep", action="store_true",
@@ -255,9 +434,12 @@ def main() -> int:
                                    "frac_hbm": round(8 * n / (ms * 1e-3) / HBM_PEAK, 4)}
 
     dom = "hom_sum_f32"
+    traffic = measured_traffic(args.kind, args.log2n, args.rel) if args.abs is None else None
     roofline = {"bound": "hbm", "kernel": dom, "achieved": ops[dom]["achieved_GBps"],
                 "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ops[dom]["frac_hbm"],
-                "traffic": MEASURED_TRAFFIC.get((args.kind, args.log2n, args.rel)) if args.abs is None else None}
+                "traffic": traffic["bytes"] if traffic and traffic["kernel"] == dom else None,
+                "traffic_calibration": traffic["calibration"] if traffic else None,
+                "traffic_source": traffic["source"] if traffic else None}
 
     out = {
         "metric": "compress + hom-add throughput (GB/s of uncompressed input)",
@@ -288,8 +470,8 @@ def main() -> int:
         torch.cuda.synchronize()
         out["error"] = error_measures(torch, x, y, dec, eb)
 
+    orc = None if args.no_cpu else entry.load_oracle()
     if not args.no_cpu:
-        orc = entry.load_oracle()
         m = min(n, 1 << args.cpu_sample_log2)
         xs, ys = x[:m].cpu().numpy(), y[:m].cpu().numpy()
         base, sa, ss = cpu_baseline(orc, xs, ys, np.float32(eb), m == n)
@@ -307,6 +489,15 @@ def main() -> int:
         if not ok:
             print(json.dumps(out))
             print("GPU streams differ from the oracle on the sample", file=sys.stderr)
+            return 1
+        del ga, gs, xs, ys, sa, ss
+    if not args.no_configs:
+        del x, y, cmp_a, cmp_b, cmp_s, dec, ws
+        torch.cuda.empty_cache()
+        out["configs"] = other_configs(torch, pkg, gen, orc)
+        if not all(c.get("matches_oracle", True) for c in out["configs"].values()):
+            print(json.dumps(out))
+            print("GPU streams differ from the oracle in one of the configurations", file=sys.stderr)
             return 1
     print(json.dumps(out))
     return 0
