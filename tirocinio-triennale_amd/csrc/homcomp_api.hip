@@ -50,8 +50,8 @@ struct homcomp_workspace {
     uint64_t *d_tile_totals;   // [max_tiles]  output-offset scan: tile totals
     uint64_t *d_tile_prefixes; // [max_tiles]  output-offset scan: tile prefixes (adjacent to the totals)
     uint64_t *d_in_ofs[2];    // [max_tiles+1] tile payload offsets of the incoming streams
-    uint32_t *d_in_totals;    // [max_tiles]   scratch of the offsets pre-pass: tile totals
-    uint32_t *d_in_blocks;    // [max_tiles/256 + 1]  and sums over blocks of 256 tiles
+    uint32_t *d_in_totals[2]; // [max_tiles]   scratch of the offsets pre-pass, per stream: tile totals
+    uint32_t *d_in_blocks[2]; // [max_tiles/256 + 1]  and sums over blocks of 256 tiles
     uint64_t *d_total;        // stream length of the last stream-producing call
     uint32_t *d_error;        // sticky error flags, next to d_total
     float *d_partial;         // min/max partials
@@ -106,14 +106,20 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
     return next_epoch(ws, s, &p->epoch);
 }
 
-// Offsets pre-pass for incoming stream c (header bytes -> payload offset of every tile).
-int in_offsets(homcomp_workspace *ws, int c, const unsigned char *d_cmp, hc::TileParams *p, hipStream_t s)
+// Offsets pre-pass of the incoming streams (header bytes -> payload offset of every tile): one
+// pass of launches for all of them.
+int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s)
 {
-    p->in_ofs[c] = ws->d_in_ofs[c];
-    return hip_ok(hc::launch_in_offsets(d_cmp, p->n_tiles, p->hdr_bytes, ws->d_in_totals, ws->d_in_blocks,
-                                        ws->d_in_ofs[c], s))
-               ? HOMCOMP_OK
-               : HOMCOMP_ERR_HIP;
+    hc::InOffsetsArgs a;
+    std::memset(&a, 0, sizeof a);
+    for (int c = 0; c < n_streams; ++c) {
+        p->in_ofs[c] = ws->d_in_ofs[c];
+        a.hdr[c] = p->in[c];
+        a.totals[c] = ws->d_in_totals[c];
+        a.block_sums[c] = ws->d_in_blocks[c];
+        a.ofs[c] = ws->d_in_ofs[c];
+    }
+    return hip_ok(hc::launch_in_offsets(a, n_streams, p->n_tiles, p->hdr_bytes, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
 // LDS stage per data wave (two deferred tiles by default), in three budgets that let 4, 3 and 2
@@ -415,8 +421,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     const size_t o_status = take(2 * t * sizeof(uint64_t));
     const size_t o_in0 = take((t + 1) * sizeof(uint64_t));
     const size_t o_in1 = take((t + 1) * sizeof(uint64_t));
-    const size_t o_tot = take(t * sizeof(uint32_t));
-    const size_t o_blk = take((t / 256 + 1) * sizeof(uint32_t));
+    const size_t o_tot0 = take(t * sizeof(uint32_t));
+    const size_t o_tot1 = take(t * sizeof(uint32_t));
+    const size_t o_blk0 = take((t / 256 + 1) * sizeof(uint32_t));
+    const size_t o_blk1 = take((t / 256 + 1) * sizeof(uint32_t));
     const size_t o_total = take(64);
     const size_t o_partial = take(kRangePartials * 2 * sizeof(float));
     const size_t bytes = off;
@@ -487,8 +495,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     ws->d_tile_prefixes = ws->d_tile_totals + t;
     ws->d_in_ofs[0] = (uint64_t *)(base + o_in0);
     ws->d_in_ofs[1] = (uint64_t *)(base + o_in1);
-    ws->d_in_totals = (uint32_t *)(base + o_tot);
-    ws->d_in_blocks = (uint32_t *)(base + o_blk);
+    ws->d_in_totals[0] = (uint32_t *)(base + o_tot0);
+    ws->d_in_totals[1] = (uint32_t *)(base + o_tot1);
+    ws->d_in_blocks[0] = (uint32_t *)(base + o_blk0);
+    ws->d_in_blocks[1] = (uint32_t *)(base + o_blk1);
     ws->d_total = (uint64_t *)(base + o_total);
     ws->d_error = (uint32_t *)(base + o_total + 8);
     ws->d_partial = (float *)(base + o_partial);
@@ -568,7 +578,7 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
     p.out_f32 = d_out;
     p.eb = eb;
     p.recip = 0.5f / eb;
-    if ((rc = in_offsets(ws, 0, d_cmp, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
     return run_tile_op(ws, hc::kOpDecompress, p, 0, s);
 }
 
@@ -592,7 +602,7 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
     return run_tile_op(ws, hc::kOpHomSumF32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
@@ -613,7 +623,7 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.local = d_local_delta;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 0, d_cmp_in, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
     return run_tile_op(ws, hc::kOpHomSumI32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
@@ -634,8 +644,7 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
     p.in_size[1] = size_b;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 0, d_cmp_a, &p, s))) return rc;
-    if ((rc = in_offsets(ws, 1, d_cmp_b, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 2, &p, s))) return rc;
     const uint64_t ta = tile_bytes_of(p, size_a), tb = tile_bytes_of(p, size_b);
     return run_tile_op(ws, hc::kOpHomAdd, p, ta > tb ? ta : tb, s);
 }
@@ -686,9 +695,13 @@ int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size
     if (!hip_ok(hc::launch_fill_u64(p.tile_totals, p.n_tiles, s)) ||
         !hip_ok(hc::launch_fill_u64(p.tile_prefixes, p.n_tiles, s)))
         return HOMCOMP_ERR_HIP;
-    if (!hip_ok(hc::launch_in_offsets(d_cmp_in, p.n_tiles, p.hdr_bytes, (uint32_t *)(base + kStaticOfsTotals),
-                                      (uint32_t *)(base + kStaticOfsBlocks), (uint64_t *)(base + kStaticOfsIn), s)))
-        return HOMCOMP_ERR_HIP;
+    hc::InOffsetsArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.hdr[0] = d_cmp_in;
+    a.totals[0] = (uint32_t *)(base + kStaticOfsTotals);
+    a.block_sums[0] = (uint32_t *)(base + kStaticOfsBlocks);
+    a.ofs[0] = (uint64_t *)(base + kStaticOfsIn);
+    if (!hip_ok(hc::launch_in_offsets(a, 1, p.n_tiles, p.hdr_bytes, s))) return HOMCOMP_ERR_HIP;
     return chained_launch(device, nullptr, 0, hc::kOpHomSumF32, p, st->grid[cls], s);
 }
 

@@ -446,25 +446,42 @@ struct SlicedIn {
     uint32_t a0, sign, ob, pl[kSlicedMaxF];
 };
 
-// The lane's block of an incoming stream from the LDS stage (`p0` = the block's first byte);
-// digest 0 (no payload, or not to be read) gives a block of zeros.
-template <uint32_t NP>   // planes that any block of the wave can have (the others are left zero without being read)
-__device__ __forceinline__ void sliced_read(const uint8_t *stage, uint32_t p0, uint32_t digest, SlicedIn &b)
+// The lane's block of an incoming stream straight from memory, as unaligned 32-bit words through a
+// range-checked buffer descriptor (`rs` starts at the tile's payload, `ofs` is the block's offset
+// in it): outlier bytes, sign word, NP planes.  A block that is not to be read (digest 0) asks
+// for words beyond every buffer and gets zeros without touching memory.  Request and use are
+// separate so that the words travel while the wave does something else.
+constexpr uint32_t kSlicedNoRead = 0xffffff00u;
+
+struct SlicedRaw {
+    uint32_t first, sign, pl[kSlicedMaxF];
+};
+
+template <uint32_t NP>   // planes that any block of the wave can have (the others are not asked for)
+__device__ __forceinline__ void sliced_request(__amdgpu_buffer_rsrc_t rs, uint32_t ofs, uint32_t digest, SlicedRaw &w)
+{
+    const uint32_t ob = digest >> 5;
+    const uint32_t at = digest ? ofs : kSlicedNoRead;
+    w.first = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)at, 0, 0);
+    w.sign = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)(at + ob), 0, 0);
+#pragma unroll
+    for (uint32_t q = 0; q < NP; ++q) w.pl[q] = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)(at + ob), (int)(4u + 4u * q), 0);
+#pragma unroll
+    for (uint32_t q = NP; q < kSlicedMaxF; ++q) w.pl[q] = 0u;   // every word has a value on every path: the struct stays in registers
+}
+
+template <uint32_t NP>
+__device__ __forceinline__ void sliced_take(const SlicedRaw &w, uint32_t digest, SlicedIn &b)
 {
     const uint32_t F = digest & 0x1fu;
     b.ob = digest >> 5;
-    const uint32_t first = load_u32_any(stage + p0);
     const uint32_t low_bytes = ~(0xffffff00u << ((8u * (b.ob - 1u)) & 31u));   // ob = 1..4
-    b.a0 = b.ob ? first & low_bytes : 0u;
-    const uint32_t sign = load_u32_any(stage + p0 + b.ob);
-    b.sign = digest ? sign : 0u;
+    b.a0 = b.ob ? w.first & low_bytes : 0u;
+    b.sign = w.sign;
 #pragma unroll
     for (uint32_t q = 0; q < kSlicedMaxF; ++q) b.pl[q] = 0u;
 #pragma unroll
-    for (uint32_t q = 0; q < NP; ++q) {
-        const uint32_t w = load_u32_any(stage + p0 + b.ob + 4u + 4u * q);
-        b.pl[q] = q < F ? w : 0u;
-    }
+    for (uint32_t q = 0; q < NP; ++q) b.pl[q] = q < F ? w.pl[q] : 0u;
 }
 
 struct SlicedOut {

@@ -246,8 +246,6 @@ __device__ __forceinline__ void scan_server(const TileParams &p, const ScanCtx &
 // area and is copied out from there.
 constexpr int kSub = kTileBlocks / 16;
 constexpr int kInStage = 16 * kMaxBlockBytes + 96;   // one sub-step's payload range, alignment shift, read-ahead slack
-// stream (+) stream stages whole tiles of few planes for the sums in the bit-plane domain
-constexpr int kInStageTile = 3 * 1024 + 64;   // half a tile of such blocks (three 1 KiB pieces) and the words read beyond its last block
 
 template <int LOCAL>
 struct SubRegs {
@@ -336,7 +334,7 @@ struct InRegs {
 };
 
 template <int NIN, int LOCAL, int OUT>
-__global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
+__global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k_wave(const TileParams p)
 {
     constexpr bool kEnc = OUT == kOutStream;
     constexpr int kW = kWG / 64;
@@ -353,7 +351,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
     // one stage per wave: the incoming streams of a sub-step are decoded one after the other
     // stream (+) stream as a sum in the bit-plane domain, tile by tile where the tiles allow it
     constexpr bool kSliced = kEnc && NIN == 2 && LOCAL == kLocalNone;
-    __shared__ __align__(16) uint8_t s_in[kW][kSliced ? kInStageTile : (NIN > 0 ? kInStage : 16)];
+    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInStage : 16];
     __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
     __shared__ __align__(4) uint8_t s_hdr_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 4];
     __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512];     // decoder: exchange of the lanes' output pieces
@@ -468,27 +466,73 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
         const int64_t t = tile_of(r);
         load_sub<LOCAL>(loc, p.local, p.n, (uint64_t)t * kTileElems, t < n_tiles, s, lane);
     };
-    auto request_in = [&](int c, int64_t r, int b, int s, InRegs (&in)[kIn]) __attribute__((always_inline)) {
+    // (`wanted` false: nothing is read, the registers are only given a value)
+    auto request_in = [&](int c, int64_t r, int b, int s, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
         uintptr_t ga;
         uint32_t shift, nbytes, rel0;
         range_of(c, b, s, ga, shift, nbytes, rel0);
         // whole 16-byte pieces; lanes beyond the range get zeros without touching memory
         const __amdgpu_buffer_rsrc_t rs =
-            buffer_of(reinterpret_cast<const void *>(ga), tile_of(r) < n_tiles ? (nbytes + 15u) & ~15u : 0u);
+            buffer_of(reinterpret_cast<const void *>(ga), wanted && tile_of(r) < n_tiles ? (nbytes + 15u) & ~15u : 0u);
         in[c].chunk = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 0, kBufCached);
     };
-    auto request = [&](int64_t r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn]) __attribute__((always_inline)) {
+    auto request = [&](int64_t r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
         request_local(r, s, loc);
         if constexpr (NIN > 0) {
 #pragma unroll
-            for (int c = 0; c < NIN; ++c) request_in(c, r, b, s, in);
+            for (int c = 0; c < NIN; ++c) request_in(c, r, b, s, in, wanted);
         }
     };
 
+    // ---- stream (+) stream in the bit-plane domain (tiles none of whose blocks has more than
+    //      kSlicedMaxF planes): a lane reads the words of its block (outlier bytes, sign word,
+    //      planes) straight from the stream, unaligned, through a descriptor of the tile's
+    //      payload.  The words of half a tile (64 blocks) are asked for while the half before is
+    //      summed, the first half of a tile at the end of the tile before, so they travel while
+    //      the wave copies the finished tile out.
+    // Most streams this path sees have one to three planes per block: a wave none of whose blocks
+    // (of the half, either stream) has more takes the code for three.
+    constexpr uint32_t kFewer = 3;
+    SlicedRaw sl_raw[2];
+    uint32_t sl_dig[2] = {0u, 0u};
+    bool sl_fewer = false;
+    // (`wanted` false: nothing is read, the registers are only given a value, so that they are not
+    // kept alive through a tile of the general path)
+    auto sliced_request_half = [&](int b, int half, bool wanted) __attribute__((always_inline)) {
+        if constexpr (kSliced) {
+            const int blk = half * 64 + lane;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) sl_dig[c] = wanted ? (uint32_t)s_hdr_in[wave][c][b][blk] : 0u;
+            sl_fewer = __builtin_amdgcn_ballot_w64((sl_dig[0] & 0x1fu) > kFewer || (sl_dig[1] & 0x1fu) > kFewer) == 0;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const uint32_t ofs = s_ofs_in[wave][c][b][blk];
+                const uint32_t room = b ? room_ctx1[c] : room_ctx0[c];
+                const uint32_t rel_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][kSub]);
+                // a block that starts below the stated size is read in full (HomComp/src/GSZ.cu:908-911);
+                // the words asked for beyond a block's last plane end at most `reach` bytes into the tile
+                uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
+                const uint32_t reach = rel_end + 8u + 4u * kSlicedMaxF;
+                if (lim > reach) lim = reach;
+                const __amdgpu_buffer_rsrc_t pay = buffer_of(p.in[c] + (b ? start_ctx1[c] : start_ctx0[c]), lim);
+                if (sl_fewer)
+                    sliced_request<kFewer>(pay, ofs, sl_dig[c], sl_raw[c]);
+                else
+                    sliced_request<kSlicedMaxF>(pay, ofs, sl_dig[c], sl_raw[c]);
+            }
+        }
+    };
+    // 32 blocks (outlier bytes, sign word, kSlicedOutPlanes planes) must fit an empty slot: they are written at once
+    const bool sliced_ok = kSliced && p.sliced &&
+                           ((p.stage_bytes / p.out_slots) & ~15u) - 64u >= 32u * (8u + 4u * (uint32_t)kSlicedOutPlanes) + 16u;
+    // does the tile in context b take the bit-plane path?
+    auto sliced_ctx = [&](int b) __attribute__((always_inline)) { return sliced_ok && ((few_ctx >> b) & 1u) != 0; };
+
     fetch_headers(0);
     prepare(0, 0);
+    sliced_request_half(0, 0, sliced_ctx(0));
 #pragma unroll
-    for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j]);
+    for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j], !sliced_ctx(0));
 
     // Deferred tiles: a tile packed in round r is copied out in round r + D (D = p.out_slots, 2 to
     // 4): its total is published when it is packed, the prefix word is requested in round
@@ -592,75 +636,23 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                 }
                 return !direct0;
             };
-            bool sliced_tile = false;
-            if constexpr (kSliced) {
-                // 32 blocks (outlier bytes, sign word, kSlicedOutPlanes planes) must fit an empty slot: they are written at once
-                sliced_tile = p.sliced && slot_cap >= 32u * (8u + 4u * (uint32_t)kSlicedOutPlanes) + 16u &&
-                              ((few_ctx >> buf) & 1u);
-            }
+            const bool sliced_tile = sliced_ctx(buf);
             if (sliced_tile) {
                 if constexpr (kSliced) {
-                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a time.
-                    //      A half tile of blocks with at most kSlicedMaxF planes is at most 64 x 32
-                    //      bytes: three 1 KiB pieces per stream with the alignment shift.  The second
-                    //      half is requested as soon as the first has gone from the registers to LDS.
-                    uint8_t *st = s_in[wave];
-                    constexpr int kPieces = 3;
-                    static_assert(64 * (4 + 4 + 4 * (int)kSlicedMaxF) + 15 <= kPieces * 1024 && kPieces * 1024 <= kInStageTile - 64,
-                                  "a half tile fits its pieces, and the words read beyond its last block the stage");
-                    uint32_t shift_h[2], rel0_h[2];
-                    u32x4 piece[2][kPieces];
-                    auto request_half = [&](int c, int half) __attribute__((always_inline)) {
-                        // blocks 64 half .. 64 half + 63 are sub-steps 4 half .. 4 half + 3
-                        const uint32_t rel0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][4 * half]);
-                        const uint32_t rel1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][buf][4 * half + 4]);
-                        const uint32_t room = buf ? room_ctx1[c] : room_ctx0[c];
-                        const uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
-                        const uint32_t end = rel1 < lim ? rel1 : lim;
-                        const uintptr_t g0 = (uintptr_t)p.in[c] + (buf ? start_ctx1[c] : start_ctx0[c]) + rel0;
-                        const uintptr_t ga = g0 & ~(uintptr_t)15;
-                        shift_h[c] = (uint32_t)(g0 - ga);
-                        rel0_h[c] = rel0;
-                        const uint32_t nbytes = end > rel0 ? shift_h[c] + (end - rel0) : 0u;
-                        const __amdgpu_buffer_rsrc_t rs = buffer_of(reinterpret_cast<const void *>(ga), (nbytes + 15u) & ~15u);
-#pragma unroll
-                        for (int i = 0; i < kPieces; ++i)
-                            piece[c][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 1024 * i, kBufCached);
-                    };
-                    auto stage_stream = [&](int c) __attribute__((always_inline)) {
-#pragma unroll
-                        for (int i = 0; i < kPieces; ++i) *reinterpret_cast<u32x4 *>(st + (lane + 64 * i) * 16) = piece[c][i];
-                        wave_lds_fence();
-                    };
-                    // Most streams this path sees have one to three planes per block: a wave none of
-                    // whose blocks (of the half, either stream) has more takes the code for three.
-                    constexpr uint32_t kFewer = 3;
-                    auto read_block = [&](int c, int half, SlicedIn &blk, bool &fewer) __attribute__((always_inline)) {
-                        const int b = half * 64 + lane;
-                        const uint32_t digest = s_hdr_in[wave][c][buf][b];
-                        const uint32_t p0 = shift_h[c] + s_ofs_in[wave][c][buf][b] - rel0_h[c];
-                        if (__builtin_amdgcn_ballot_w64((digest & 0x1fu) > kFewer) == 0) {
-                            sliced_read<kFewer>(st, p0, digest, blk);
-                        } else {
-                            sliced_read<kSlicedMaxF>(st, p0, digest, blk);
-                            fewer = false;
-                        }
-                    };
-                    request_half(0, 0);
-                    request_half(1, 0);
+                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a time
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
                         SlicedIn A, B;
                         SlicedOut out;
-                        bool fewer = true;
-                        stage_stream(0);
-                        read_block(0, half, A, fewer);
-                        wave_lds_fence();
-                        if (half == 0) request_half(0, 1);   // after read_block: it replaces shift_h / rel0_h of the stream
-                        stage_stream(1);
-                        read_block(1, half, B, fewer);
-                        wave_lds_fence();
-                        if (half == 0) request_half(1, 1);
+                        const bool fewer = sl_fewer;
+                        if (fewer) {
+                            sliced_take<kFewer>(sl_raw[0], sl_dig[0], A);
+                            sliced_take<kFewer>(sl_raw[1], sl_dig[1], B);
+                        } else {
+                            sliced_take<kSlicedMaxF>(sl_raw[0], sl_dig[0], A);
+                            sliced_take<kSlicedMaxF>(sl_raw[1], sl_dig[1], B);
+                        }
+                        if (half == 0) sliced_request_half(buf, 1, true);   // on its way while the first half is summed
                         if (fewer)
                             sliced_add<kFewer>(A, B, out);
                         else
@@ -685,10 +677,13 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
                         }
                     }
                     wave_lds_fence();
-                    // the next tile's block offsets and first requests, as the sub-steps below leave them
+                    // the next tile's block offsets and first requests: of its first half on this
+                    // path, else as the sub-steps below leave them
                     prepare(r + 1, buf ^ 1);
+                    const bool next_sliced = tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1);
+                    sliced_request_half(buf ^ 1, 0, next_sliced);
 #pragma unroll
-                    for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j]);
+                    for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j], !next_sliced);
                 }
             } else {
             // sub-step s of this tile; (r2, b2, s2) is the sub-step the freed registers are requested for
@@ -809,6 +804,7 @@ __global__ __launch_bounds__(kWG) void k_wave(const TileParams p)
 #pragma unroll
                 for (int j = 0; j < kDepth; ++j) sub(s + j, loc[j], in[j], r + wrap, buf ^ wrap, s2 + j);
             }
+            if constexpr (kSliced) sliced_request_half(buf ^ 1, 0, tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1));
             }
             if constexpr (kEnc) {
                 wave_lds_fence();
@@ -856,11 +852,13 @@ __device__ __forceinline__ uint32_t wg_reduce_u32(uint32_t v, uint32_t *s_tmp)
 
 // A stream of at most one block of tiles (4 MiB of values) gets its offsets from k_in_totals
 // itself (`ofs` not null, one workgroup): the second launch would be a fifth of such a call.
-__global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ hdr, uint32_t n_tiles,
-                                                   uint32_t *__restrict__ totals,
-                                                   uint32_t *__restrict__ block_sums,
-                                                   uint64_t base, uint64_t *__restrict__ ofs)
+// One launch serves up to two streams (blockIdx.y), each with its own arrays.
+__global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base, int direct)
 {
+    const uint8_t *__restrict__ hdr = a.hdr[blockIdx.y];
+    uint32_t *__restrict__ totals = a.totals[blockIdx.y];
+    uint32_t *__restrict__ block_sums = a.block_sums[blockIdx.y];
+    uint64_t *__restrict__ ofs = direct ? a.ofs[blockIdx.y] : nullptr;
     __shared__ uint32_t s_tmp[4];
     __shared__ uint32_t s_tot[kOfsBlockTiles];
     uint32_t acc = 0;
@@ -924,11 +922,11 @@ __global__ __launch_bounds__(256) void k_in_totals(const uint8_t *__restrict__ h
     if (threadIdx.x == 0) ofs[n_tiles] = base + block_total;   // the end of the payload
 }
 
-__global__ __launch_bounds__(256) void k_in_offsets(const uint32_t *__restrict__ totals,
-                                                    const uint32_t *__restrict__ block_sums,
-                                                    uint32_t n_tiles, uint64_t base,
-                                                    uint64_t *__restrict__ ofs)
+__global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base)
 {
+    const uint32_t *__restrict__ totals = a.totals[blockIdx.y];
+    const uint32_t *__restrict__ block_sums = a.block_sums[blockIdx.y];
+    uint64_t *__restrict__ ofs = a.ofs[blockIdx.y];
     __shared__ uint32_t s_tmp[4];
     __shared__ uint32_t s_wave[4];
     // bytes of all earlier blocks (a block is at most 256 * 132 * 128 bytes, so 64-bit sums)
@@ -1130,17 +1128,15 @@ hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t
     }
 }
 
-hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
-                             uint32_t *block_sums, uint64_t *ofs, hipStream_t s)
+hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, hipStream_t s)
 {
     const uint32_t blocks = (n_tiles + kOfsBlockTiles - 1) / kOfsBlockTiles;
     if (blocks == 1) {
-        hipLaunchKernelGGL(k_in_totals, dim3(1), dim3(256), 0, s, hdr, n_tiles, totals, block_sums, base, ofs);
+        hipLaunchKernelGGL(k_in_totals, dim3(1, n_streams), dim3(256), 0, s, a, n_tiles, base, 1);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(k_in_totals, dim3(blocks), dim3(256), 0, s, hdr, n_tiles, totals, block_sums, (uint64_t)0,
-                       (uint64_t *)nullptr);
-    hipLaunchKernelGGL(k_in_offsets, dim3(blocks), dim3(256), 0, s, totals, block_sums, n_tiles, base, ofs);
+    hipLaunchKernelGGL(k_in_totals, dim3(blocks, n_streams), dim3(256), 0, s, a, n_tiles, (uint64_t)0, 0);
+    hipLaunchKernelGGL(k_in_offsets, dim3(blocks, n_streams), dim3(256), 0, s, a, n_tiles, base);
     return hipGetLastError();
 }
 

@@ -47,9 +47,16 @@ constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
 // Resident workgroups per compute unit of the kernel behind an operation (sizes the persistent grid).
 hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu);
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
-// Tile payload offsets of an incoming stream from its header bytes.
-hipError_t launch_in_offsets(const uint8_t *hdr, uint32_t n_tiles, uint64_t base, uint32_t *totals,
-                             uint32_t *block_sums, uint64_t *ofs, hipStream_t s);
+// Tile payload offsets of one or two incoming streams (of the same length) from their header
+// bytes, in one pass of launches: per stream the header bytes, two scratch arrays (n_tiles totals,
+// n_tiles / 256 + 1 sums) and the n_tiles + 1 offsets to be written.
+struct InOffsetsArgs {
+    const uint8_t *hdr[2];
+    uint32_t *totals[2];
+    uint32_t *block_sums[2];
+    uint64_t *ofs[2];
+};
+hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, hipStream_t s);
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s);
 hipError_t launch_range(const float *x, uint64_t n, float *partial, uint32_t max_partials,
                         float *out, hipStream_t s);
