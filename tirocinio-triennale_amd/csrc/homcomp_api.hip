@@ -131,6 +131,7 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
 // matter.  (With the full 8 KiB slots only one workgroup of the two-stream kernel
 // fits a compute unit, which is slower than spilling: its largest slots are 7.3 KiB.)
 constexpr int kStageClasses = 3;
+constexpr uint64_t kBitplaneTileBytes = hc::kHostTileBlocks * 20u;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
     {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4112 + 64)},
@@ -265,6 +266,9 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         p.stage_bytes = 0u;
         return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
+    // stream (+) local operand: the kernel with the bit-plane path where the incoming blocks can
+    // have the few planes it takes (at most 4 + 4 * 3 + 4 bytes each on average), else the one without
+    if ((op == hc::kOpHomSumF32 || op == hc::kOpHomSumI32) && expected_tile_bytes > kBitplaneTileBytes) p.sliced = 0;
     if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
     int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
     if (ws->stage_class >= 0) cls = ws->stage_class;
@@ -688,7 +692,7 @@ int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size
     p.recip = 0.5f / eb;
     p.spill = base + kStaticOfsSpill;
     p.out_slots = kStaticSlots;
-    p.sliced = 1;
+    p.sliced = tile_bytes_of(p, cmp_in_size) <= kBitplaneTileBytes;
     const int cls = choose_stage_class(hc::kOpHomSumF32, tile_bytes_of(p, cmp_in_size), kStaticSlots);
     p.stage_bytes = kStage[cls][hc::kOpHomSumF32];
     // totals and prefixes of the tiles this call uses (the arrays keep the last call's words)

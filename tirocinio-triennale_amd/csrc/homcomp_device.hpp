@@ -434,6 +434,12 @@ __device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0,
 // out as they came in.
 constexpr uint32_t kSlicedMaxF = 6;
 constexpr int kSlicedOutPlanes = kSlicedMaxF + 2;   // plain mode can take element 0 one plane further
+// The common streams have one to three planes per block: code for kFewPlanes serves waves none
+// of whose blocks has more.  stream (+) local operand takes the bit-plane path for such tiles
+// only, with the local deltas as kLocalFew two's-complement planes (sign plane included), so a
+// sum has up to kLocalFew + 1 bits.
+constexpr uint32_t kFewPlanes = 3, kLocalFew = 4;
+constexpr int kSlicedOutWords = kSlicedOutPlanes > (int)kLocalFew + 1 ? kSlicedOutPlanes : (int)kLocalFew + 1;
 
 typedef uint32_t __attribute__((aligned(1))) u32_unaligned;
 __device__ __forceinline__ uint32_t load_u32_any(const uint8_t *p) { return *reinterpret_cast<const u32_unaligned *>(p); }
@@ -485,8 +491,36 @@ __device__ __forceinline__ void sliced_take(const SlicedRaw &w, uint32_t digest,
 }
 
 struct SlicedOut {
-    uint32_t hdr, size, ob, F, a0, sign, m[kSlicedOutPlanes];
+    uint32_t hdr, size, ob, F, a0, sign, m[kSlicedOutWords];
 };
+
+// Rate selection of a block summed in the bit-plane domain (HomComp/src/GSZ.cu:151-167): `nz` has
+// bit q set when magnitude plane q of elements 1..31 is not empty, s0 is the sum of element 0,
+// `sign` the sign plane of elements 1..31; o.m[] holds the magnitude planes, o.a0 = |s0|.
+template <uint32_t NW>   // words of o.m[] a block can need
+__device__ __forceinline__ void sliced_select(uint32_t nz, uint32_t s0, uint32_t sign, SlicedOut &o)
+{
+    constexpr uint32_t E = 0x80u;   // element 0
+    const uint32_t fr2 = bit_num(nz);                      // elements 1..31   (:153)
+    const uint32_t b0 = bit_num(o.a0);
+    uint32_t fr1 = b0 > fr2 ? b0 : fr2;                    // all 32 elements  (:152)
+    if (fr1 > 31u) fr1 = 31u;
+    const uint32_t ob = (b0 + 7u) >> 3;                    // :154
+    const uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;         // :156
+    const uint32_t sz2 = 4u + 4u * fr2 + ob;               // :157
+    const bool plain = sz1 <= sz2;                         // :158-164
+    o.hdr = plain ? fr1 : fr2 | 0x80u | ((ob - 1u) << 5);
+    o.size = plain ? sz1 : sz2;
+    o.F = plain ? fr1 : fr2;
+    o.ob = plain ? 0u : ob;
+    o.sign = sign | (((int32_t)s0 < 0) ? E : 0u);
+    // plain mode: element 0 goes back into the planes (it has at most one plane more than the rest)
+    const uint32_t ins = plain ? o.a0 : 0u;
+    if (__builtin_amdgcn_ballot_w64(ins != 0u) != 0) {
+#pragma unroll
+        for (uint32_t q = 0; q < NW; ++q) o.m[q] |= ((ins >> q) & 1u) << 7;
+    }
+}
 
 // delta_out = delta_A + delta_B for the lane's block, and the block's rate selection
 // (HomComp/src/GSZ.cu:151-167).
@@ -535,7 +569,7 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
     const uint32_t SR = r[NP + 1];   // the sign plane: the sums fit NP + 1 bits
     uint32_t c = SR, nz = 0;
 #pragma unroll
-    for (uint32_t q = 0; q < kSlicedOutPlanes; ++q) o.m[q] = 0;
+    for (uint32_t q = 0; q < (uint32_t)kSlicedOutWords; ++q) o.m[q] = 0;
 #pragma unroll
     for (uint32_t q = 0; q < NP + 1; ++q) {
         const uint32_t t = r[q] ^ SR;
@@ -543,38 +577,106 @@ __device__ __forceinline__ void sliced_add(const SlicedIn &A, const SlicedIn &B,
         c &= t;
         nz |= (o.m[q] ? 1u : 0u) << q;
     }
-    // ---- rate selection
-    const uint32_t fr2 = bit_num(nz);                      // elements 1..31   (:153)
-    const uint32_t b0 = bit_num(o.a0);
-    uint32_t fr1 = b0 > fr2 ? b0 : fr2;                    // all 32 elements  (:152)
-    if (fr1 > 31u) fr1 = 31u;
-    const uint32_t ob = (b0 + 7u) >> 3;                    // :154
-    const uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;         // :156
-    const uint32_t sz2 = 4u + 4u * fr2 + ob;               // :157
-    const bool plain = sz1 <= sz2;                         // :158-164
-    o.hdr = plain ? fr1 : fr2 | 0x80u | ((ob - 1u) << 5);
-    o.size = plain ? sz1 : sz2;
-    o.F = plain ? fr1 : fr2;
-    o.ob = plain ? 0u : ob;
-    o.sign = SR | (((int32_t)s0 < 0) ? E : 0u);
-    // plain mode: element 0 goes back into the planes (it has at most one plane more than the rest)
-    const uint32_t ins = plain ? o.a0 : 0u;
-    if (__builtin_amdgcn_ballot_w64(ins != 0u) != 0) {
+    sliced_select<NP + 2>(nz, s0, SR, o);
+}
+
+// delta_out = delta_A + delta_local for the lane's block: A from a stream (sign and magnitude
+// planes, NPA of them), the local deltas as NPB two's-complement planes `plB` (the last one is the
+// sign plane; element 0's bit is clear in all of them) with the delta of element 0 beside them
+// in b0 (HomComp/src/homcomp.cu:3601-3660 computes the same sums value by value).
+template <uint32_t NPA, uint32_t NPB>
+__device__ __forceinline__ void sliced_add_local(const SlicedIn &A, const uint32_t (&plB)[NPB], uint32_t b0, SlicedOut &o)
+{
+    constexpr uint32_t E = 0x80u;   // element 0
+    constexpr uint32_t W = (NPA + 1 > NPB ? NPA + 1 : NPB) + 1;   // bits of a sum, sign included
+    static_assert(W <= (uint32_t)kSlicedOutWords, "the sums fit the output planes");
+    // ---- element 0: plane bits in plain mode, the outlier in outlier mode
+    uint32_t m0A = A.a0;
+    {
+        uint32_t anyA = 0;
 #pragma unroll
-        for (uint32_t q = 0; q < NP + 2; ++q) o.m[q] |= ((ins >> q) & 1u) << 7;
+        for (uint32_t q = 0; q < NPA; ++q) anyA |= A.pl[q];
+        const bool gatherA = A.ob == 0u && (anyA & E);
+        if (__builtin_amdgcn_ballot_w64(gatherA) != 0) {   // wave-uniform; rare where outlier mode prevails
+            uint32_t gA = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < NPA; ++q) gA |= ((A.pl[q] >> 7) & 1u) << q;
+            if (A.ob == 0u) m0A = gA;
+        }
     }
+    const uint32_t v0A = (A.sign & E) ? 0u - m0A : m0A;
+    const uint32_t s0 = v0A + b0;   // wrapping, as the reference's int
+    const int32_t s0neg = (int32_t)(0u - s0);
+    o.a0 = (uint32_t)((int32_t)s0 > s0neg ? (int32_t)s0 : s0neg);   // |s0| (0x80000000 stays)
+    // ---- elements 1..31, plane by plane
+    const uint32_t SA = A.sign & ~E;
+    uint32_t cA = SA, carry = 0, r[W];
+#pragma unroll
+    for (uint32_t q = 0; q < W; ++q) {
+        const uint32_t tA = (q < NPA ? A.pl[q] & ~E : 0u) ^ SA;
+        const uint32_t xA = tA ^ cA;
+        cA &= tA;
+        const uint32_t xB = plB[q < NPB ? q : NPB - 1];
+        r[q] = xA ^ xB ^ carry;
+        carry = (xA & xB) | (carry & (xA ^ xB));
+    }
+    const uint32_t SR = r[W - 1];   // the sign plane
+    uint32_t c = SR, nz = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < (uint32_t)kSlicedOutWords; ++q) o.m[q] = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < W - 1; ++q) {
+        const uint32_t t = r[q] ^ SR;
+        o.m[q] = t ^ c;
+        c &= t;
+        nz |= (o.m[q] ? 1u : 0u) << q;
+    }
+    sliced_select<W>(nz, s0, SR, o);
+}
+
+// The local operand of a sub-step (16 blocks, 8 deltas per lane, 4 lanes per block) as
+// two's-complement planes: lane k of a quad ends up with the whole word of plane k of its block.  Plane bytes come out of the same bit-matrix transposition as in pack8 (a
+// lane's byte of a plane covers its 8 elements, element 0 of the lane at the top bit); the four
+// bytes of a word are then collected across the quad with two lane exchanges.
+// sel1 / sel2: the lane's byte selectors of the two exchanges (quad_transpose_selectors).
+__device__ __forceinline__ void quad_transpose_selectors(int k, uint32_t &sel1, uint32_t &sel2)
+{
+    sel1 = (k & 1) ? 0x03070105u : 0x06020400u;   // odd lanes keep bytes 1, 3 and take the partner's; even lanes bytes 0, 2
+    sel2 = (k & 2) ? 0x03020706u : 0x05040100u;   // lanes 2, 3 keep the upper half word, lanes 0, 1 the lower
+}
+
+// y: byte p = the lane's byte (number k) of plane p's word.  Returns the word of plane k.
+__device__ __forceinline__ uint32_t quad_transpose_bytes(uint32_t y, uint32_t sel1, uint32_t sel2)
+{
+    const uint32_t t = dpp_u32<kDppXor1>(y);
+    const uint32_t u = __builtin_amdgcn_perm(t, y, sel1);
+    const uint32_t t2 = dpp_u32<kDppXor2>(u);
+    return __builtin_amdgcn_perm(t2, u, sel2);
+}
+
+// Four planes of deltas within -8 .. 7.
+__device__ __forceinline__ uint32_t local_planes4(const int32_t v[8], uint32_t sel1, uint32_t sel2)
+{
+    constexpr uint32_t two = 0x0c0c0400u;
+    const uint32_t lo = __builtin_amdgcn_perm(__builtin_amdgcn_perm((uint32_t)v[4], (uint32_t)v[5], two),
+                                              __builtin_amdgcn_perm((uint32_t)v[6], (uint32_t)v[7], two), 0x05040100u);
+    const uint32_t hi = __builtin_amdgcn_perm(__builtin_amdgcn_perm((uint32_t)v[0], (uint32_t)v[1], two),
+                                              __builtin_amdgcn_perm((uint32_t)v[2], (uint32_t)v[3], two), 0x05040100u);
+    // low nibbles of lo, low nibbles of hi moved up: (lo & 0x0f0f0f0f) | ((hi << 4) & 0xf0f0f0f0)
+    const uint32_t y = transpose4((lo & 0x0f0f0f0fu) | ((hi << 4) & 0xf0f0f0f0u));
+    return quad_transpose_bytes(y, sel1, sel2);
 }
 
 // The block's payload at `pos` of the stage: outlier bytes (a whole word is stored; what it
 // writes beyond them is overwritten by the sign word), sign word, planes.
-template <uint32_t NP>
+template <uint32_t NW>   // plane words a block of the wave can have
 __device__ __forceinline__ void sliced_write(lds_bytes stage, uint32_t pos, const SlicedOut &o)
 {
     if (o.hdr == 0u) return;
     if (o.ob) store_u32_any(stage + pos, o.a0);
     store_u32_any(stage + pos + o.ob, o.sign);
 #pragma unroll
-    for (uint32_t q = 0; q < NP + 2; ++q)
+    for (uint32_t q = 0; q < NW; ++q)
         if (q < o.F) store_u32_any(stage + pos + o.ob + 4u + 4u * q, o.m[q]);
 }
 

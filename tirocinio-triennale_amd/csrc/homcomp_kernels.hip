@@ -9,6 +9,9 @@
 #include "homcomp_device.hpp"
 #include "homcomp_kernels.hpp"
 
+#ifndef HC_LOAD_POLICY
+#define HC_LOAD_POLICY 0
+#endif
 #ifndef HC_DEPTH_ENC
 #define HC_DEPTH_ENC 2
 #endif
@@ -261,8 +264,8 @@ __device__ __forceinline__ void load_sub(SubRegs<LOCAL> &r, const void *local, u
     if constexpr (LOCAL == kLocalNone) return;
     const uint64_t left = valid && tile_elem0 < n ? (n - tile_elem0) * 4u : 0u;
     const __amdgpu_buffer_rsrc_t rs = buffer_of((const uint8_t *)local + (valid ? tile_elem0 * 4u : 0u), left);
-    const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32, s * 2048, kBufNt);
-    const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32 + 16, s * 2048, kBufNt);
+    const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32, s * 2048, HC_LOAD_POLICY);
+    const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 32 + 16, s * 2048, HC_LOAD_POLICY);
     if constexpr (LOCAL == kLocalF32) {
         r.f[0] = __builtin_bit_cast(f32x4, a);
         r.f[1] = __builtin_bit_cast(f32x4, b);
@@ -333,7 +336,10 @@ struct InRegs {
     u32x4 chunk;   // the lane's 16-byte chunk of a sub-step's payload range
 };
 
-template <int NIN, int LOCAL, int OUT>
+// BITPLANE: the kernel has the bit-plane paths.  stream (+) local operand comes in both kinds: the
+// host launches the kind without them where the incoming stream is too wide for them anyway,
+// because the general path alone is the faster code for such data (fewer registers in use).
+template <int NIN, int LOCAL, int OUT, bool BITPLANE>
 __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k_wave(const TileParams p)
 {
     constexpr bool kEnc = OUT == kOutStream;
@@ -350,8 +356,15 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
     // one stage per wave: the incoming streams of a sub-step are decoded one after the other
     // stream (+) stream as a sum in the bit-plane domain, tile by tile where the tiles allow it
-    constexpr bool kSliced = kEnc && NIN == 2 && LOCAL == kLocalNone;
-    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInStage : 16];
+    constexpr bool kSliced = BITPLANE && kEnc && NIN == 2 && LOCAL == kLocalNone;
+    // stream (+) local operand likewise, the local deltas turned into bit planes on the way
+    constexpr bool kSlicedLocal = BITPLANE && kEnc && NIN == 1 && LOCAL != kLocalNone;
+    constexpr bool kAnySliced = kSliced || kSlicedLocal;
+    // the planes of the local operand of half a tile, a row of 64 words per plane and one for the
+    // deltas of the blocks' first elements; they share the wave's stage of incoming payload
+    constexpr int kLocalRows = (int)kLocalFew + 1;
+    constexpr int kInBytes = kSlicedLocal && kLocalRows * 256 > kInStage ? kLocalRows * 256 : kInStage;
+    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInBytes : 16];
     __shared__ __align__(4) uint16_t s_ofs_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 2];
     __shared__ __align__(4) uint8_t s_hdr_in[kW][kIn][2][NIN > 0 ? kTileBlocks : 4];
     __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512];     // decoder: exchange of the lanes' output pieces
@@ -384,7 +397,8 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     // bytes of the stream from the tile's payload start to its stated end, saturated to 32 bits:
     // everything inside a tile is 32-bit arithmetic against these
     uint32_t room_ctx0[kIn], room_ctx1[kIn];
-    uint32_t few_ctx = 0;   // kSliced: bit b set = no block of the tile in context b (either stream) has more than kSlicedMaxF planes
+    uint32_t end_ctx0[kIn], end_ctx1[kIn];   // payload bytes of those tiles
+    uint32_t few_ctx = 0;   // bit-plane paths: bit b set = the blocks of the tile in context b (any stream) have few enough planes for them
     auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             int64_t t = tile_of(r);
@@ -420,18 +434,23 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     const uint32_t d0 = z0 != 0u && o0 < room ? header_digest(h0) : 0u;
                     const uint32_t d1 = z1 != 0u && o1 < room ? header_digest(h1) : 0u;
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
-                    if constexpr (kSliced) {
-                        const bool few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > kSlicedMaxF || (d1 & 0x1fu) > kSlicedMaxF) == 0;
+                    if constexpr (kAnySliced) {
+                        // stream (+) stream takes tiles of up to kSlicedMaxF planes, stream (+) local operand of up to kFewPlanes
+                        constexpr uint32_t most = kSliced ? kSlicedMaxF : kFewPlanes;
+                        const bool few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > most || (d1 & 0x1fu) > most) == 0;
                         const uint32_t bit = 1u << b;
                         if (c == 0) few_ctx |= bit;
                         if (!few) few_ctx &= ~bit;
                     }
+                    const uint32_t tile_end = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     if (b) {
                         start_ctx1[c] = start_next[c];
                         room_ctx1[c] = room;
+                        end_ctx1[c] = tile_end;
                     } else {
                         start_ctx0[c] = start_next[c];
                         room_ctx0[c] = room;
+                        end_ctx0[c] = tile_end;
                     }
                 }
                 wave_lds_fence();
@@ -492,23 +511,27 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     //      the wave copies the finished tile out.
     // Most streams this path sees have one to three planes per block: a wave none of whose blocks
     // (of the half, either stream) has more takes the code for three.
-    constexpr uint32_t kFewer = 3;
-    SlicedRaw sl_raw[2];
-    uint32_t sl_dig[2] = {0u, 0u};
+    constexpr uint32_t kFewer = kFewPlanes;
+    SlicedRaw sl_raw[kIn];
+    uint32_t sl_dig[kIn];
     bool sl_fewer = false;
     // (`wanted` false: nothing is read, the registers are only given a value, so that they are not
     // kept alive through a tile of the general path)
     auto sliced_request_half = [&](int b, int half, bool wanted) __attribute__((always_inline)) {
-        if constexpr (kSliced) {
+        if constexpr (kAnySliced) {
             const int blk = half * 64 + lane;
+            bool more = false;
 #pragma unroll
-            for (int c = 0; c < 2; ++c) sl_dig[c] = wanted ? (uint32_t)s_hdr_in[wave][c][b][blk] : 0u;
-            sl_fewer = __builtin_amdgcn_ballot_w64((sl_dig[0] & 0x1fu) > kFewer || (sl_dig[1] & 0x1fu) > kFewer) == 0;
+            for (int c = 0; c < NIN; ++c) {
+                sl_dig[c] = wanted ? (uint32_t)s_hdr_in[wave][c][b][blk] : 0u;
+                more = more || (sl_dig[c] & 0x1fu) > kFewer;
+            }
+            sl_fewer = __builtin_amdgcn_ballot_w64(more) == 0;
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
+            for (int c = 0; c < NIN; ++c) {
                 const uint32_t ofs = s_ofs_in[wave][c][b][blk];
                 const uint32_t room = b ? room_ctx1[c] : room_ctx0[c];
-                const uint32_t rel_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_rel[wave][c][b][kSub]);
+                const uint32_t rel_end = b ? end_ctx1[c] : end_ctx0[c];
                 // a block that starts below the stated size is read in full (HomComp/src/GSZ.cu:908-911);
                 // the words asked for beyond a block's last plane end at most `reach` bytes into the tile
                 uint32_t lim = room ? room + (kMaxBlockBytes - 1) : 0u;
@@ -522,11 +545,21 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             }
         }
     };
-    // 32 blocks (outlier bytes, sign word, kSlicedOutPlanes planes) must fit an empty slot: they are written at once
-    const bool sliced_ok = kSliced && p.sliced &&
-                           ((p.stage_bytes / p.out_slots) & ~15u) - 64u >= 32u * (8u + 4u * (uint32_t)kSlicedOutPlanes) + 16u;
+    // 32 blocks (outlier bytes, sign word, planes) must fit an empty slot: they are written at once
+    constexpr uint32_t kSlicedWords = kSlicedLocal ? kLocalFew + 1u : (uint32_t)kSlicedOutPlanes;
+    const bool sliced_ok = kAnySliced && p.sliced &&
+                           ((p.stage_bytes / p.out_slots) & ~15u) - 64u >= 32u * (8u + 4u * kSlicedWords) + 16u;
+    // The local operand is only known to fit its planes (deltas within -8 .. 7) once it has been
+    // quantised.  A tile goes down the bit-plane path when its incoming blocks have few planes
+    // and the tile before gave no reason for doubt: a half tile whose local deltas did not fit is
+    // redone by the general path and withdraws the trust, a tile of the general path whose sums
+    // all have few planes restores it.
+    bool sl_trust = true;
+    uint32_t planes_seen = 0;   // general path: the largest plane count among the lane's output blocks of the tile
     // does the tile in context b take the bit-plane path?
-    auto sliced_ctx = [&](int b) __attribute__((always_inline)) { return sliced_ok && ((few_ctx >> b) & 1u) != 0; };
+    auto sliced_ctx = [&](int b) __attribute__((always_inline)) { return sliced_ok && sl_trust && ((few_ctx >> b) & 1u) != 0; };
+    uint32_t sel1 = 0, sel2 = 0;
+    if constexpr (kSlicedLocal) quad_transpose_selectors(k, sel1, sel2);
 
     fetch_headers(0);
     prepare(0, 0);
@@ -636,70 +669,10 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                 }
                 return !direct0;
             };
-            const bool sliced_tile = sliced_ctx(buf);
-            if (sliced_tile) {
-                if constexpr (kSliced) {
-                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a time
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        SlicedIn A, B;
-                        SlicedOut out;
-                        const bool fewer = sl_fewer;
-                        if (fewer) {
-                            sliced_take<kFewer>(sl_raw[0], sl_dig[0], A);
-                            sliced_take<kFewer>(sl_raw[1], sl_dig[1], B);
-                        } else {
-                            sliced_take<kSlicedMaxF>(sl_raw[0], sl_dig[0], A);
-                            sliced_take<kSlicedMaxF>(sl_raw[1], sl_dig[1], B);
-                        }
-                        if (half == 0) sliced_request_half(buf, 1, true);   // on its way while the first half is summed
-                        if (fewer)
-                            sliced_add<kFewer>(A, B, out);
-                        else
-                            sliced_add<kSlicedMaxF>(A, B, out);
-                        s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
-                        const uint32_t incl = wave_incl_scan_u32(out.size, lane);
-                        const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
-                        const uint32_t all64 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
-                        // two writes of 32 blocks each, so that what is written at once fits an empty slot
-#pragma unroll
-                        for (int q = 0; q < 2; ++q) {
-                            const uint32_t bytes = q ? all64 - first32 : first32;
-                            make_room(bytes);   // always true here: 32 blocks fit an empty slot
-                            const uint32_t pos = run - flushed + (incl - out.size) - (q ? first32 : 0u);
-                            if ((lane >> 5) == q) {
-                                if (fewer)
-                                    sliced_write<kFewer>((lds_bytes)stage, pos, out);
-                                else
-                                    sliced_write<kSlicedMaxF>((lds_bytes)stage, pos, out);
-                            }
-                            run += bytes;
-                        }
-                    }
-                    wave_lds_fence();
-                    // the next tile's block offsets and first requests: of its first half on this
-                    // path, else as the sub-steps below leave them
-                    prepare(r + 1, buf ^ 1);
-                    const bool next_sliced = tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1);
-                    sliced_request_half(buf ^ 1, 0, next_sliced);
-#pragma unroll
-                    for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j], !next_sliced);
-                }
-            } else {
             // sub-step s of this tile; (r2, b2, s2) is the sub-step the freed registers are requested for
-            auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2) __attribute__((always_inline)) {
-                // the blocks' digests and offsets first: nothing in the sub-step writes them, and
-                // read here they are on their way while the wave waits for its operands
-                uint32_t digest[kIn], ofs[kIn];
-                if constexpr (NIN > 0) {
-#pragma unroll
-                    for (int c = 0; c < NIN; ++c) {
-                        digest[c] = s_hdr_in[wave][c][buf][s * 16 + quad];
-                        ofs[c] = s_ofs_in[wave][c][buf][s * 16 + quad];
-                    }
-                }
-                // elements beyond the end arrive as zeros (0.0f quantises to 0), as the reference pads
-                int32_t v[8];
+            // the lane's eight local deltas of a sub-step from its operand registers;
+            // elements beyond the end arrive as zeros (0.0f quantises to 0), as the reference pads
+            auto local_deltas = [&](const SubRegs<LOCAL> &loc, int32_t (&v)[8]) __attribute__((always_inline)) {
                 if constexpr (LOCAL == kLocalF32) {
                     // HomComp/src/GSZ.cu:82-149: quantise, Lorenzo with prevQuant = 0 at block start
                     const float x[8] = {loc.f[0].x, loc.f[0].y, loc.f[0].z, loc.f[0].w,
@@ -720,7 +693,23 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
                     for (int m = 0; m < 8; ++m) v[m] = 0;
                 }
-                request_local(r2, s2, loc);
+            };
+            // `ahead` false: the registers are not sent out again (a sub-step run out of turn)
+            auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2, bool ahead = true)
+                           __attribute__((always_inline)) {
+                // the blocks' digests and offsets first: nothing in the sub-step writes them, and
+                // read here they are on their way while the wave waits for its operands
+                uint32_t digest[kIn], ofs[kIn];
+                if constexpr (NIN > 0) {
+#pragma unroll
+                    for (int c = 0; c < NIN; ++c) {
+                        digest[c] = s_hdr_in[wave][c][buf][s * 16 + quad];
+                        ofs[c] = s_ofs_in[wave][c][buf][s * 16 + quad];
+                    }
+                }
+                int32_t v[8];
+                local_deltas(loc, v);
+                if (ahead) request_local(r2, s2, loc);
                 if constexpr (NIN > 0) {
 #pragma unroll
                     for (int c = 0; c < NIN; ++c) {
@@ -738,7 +727,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                                 *reinterpret_cast<u32x4 *>(st + 16u * i) =
                                     __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(16u * i), 0, kBufCached);
                         }
-                        request_in(c, r2, b2, s2, in);
+                        if (ahead) request_in(c, r2, b2, s2, in);
                         wave_lds_fence();
                         // ---- decode (HomComp/src/GSZ.cu:883-1434)
                         unpack8_add(st, shift + ofs[c] - rel0, digest[c], k, v);
@@ -786,6 +775,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     const uint32_t incl = quad_incl_scan_u32(size);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
+                    if constexpr (kSlicedLocal) planes_seen = planes_seen > (hd & 0x1fu) ? planes_seen : (hd & 0x1fu);
                     make_room(sub_total);
                     if (direct0)
                         pack8((global_bytes)slot, run + incl - size, hd, k, a, sb, a0);
@@ -794,6 +784,141 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     run += sub_total;
                 }
             };
+            const bool sliced_tile = sliced_ctx(buf);
+            if (sliced_tile) {
+                if constexpr (kSliced) {
+                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a time
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        SlicedIn A, B;
+                        SlicedOut out;
+                        const bool fewer = sl_fewer;
+                        if (fewer) {
+                            sliced_take<kFewer>(sl_raw[0], sl_dig[0], A);
+                            sliced_take<kFewer>(sl_raw[1], sl_dig[1], B);
+                        } else {
+                            sliced_take<kSlicedMaxF>(sl_raw[0], sl_dig[0], A);
+                            sliced_take<kSlicedMaxF>(sl_raw[1], sl_dig[1], B);
+                        }
+                        if (half == 0) sliced_request_half(buf, 1, true);   // on its way while the first half is summed
+                        if (fewer)
+                            sliced_add<kFewer>(A, B, out);
+                        else
+                            sliced_add<kSlicedMaxF>(A, B, out);
+                        s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
+                        const uint32_t incl = wave_incl_scan_u32(out.size, lane);
+                        const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
+                        const uint32_t all64 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+                        // two writes of 32 blocks each, so that what is written at once fits an empty slot
+#pragma unroll
+                        for (int q = 0; q < 2; ++q) {
+                            const uint32_t bytes = q ? all64 - first32 : first32;
+                            make_room(bytes);   // always true here: 32 blocks fit an empty slot
+                            const uint32_t pos = run - flushed + (incl - out.size) - (q ? first32 : 0u);
+                            if ((lane >> 5) == q) {
+                                if (fewer)
+                                    sliced_write<kFewer + 2>((lds_bytes)stage, pos, out);
+                                else
+                                    sliced_write<kSlicedMaxF + 2>((lds_bytes)stage, pos, out);
+                            }
+                            run += bytes;
+                        }
+                    }
+                    wave_lds_fence();
+                    // the next tile's block offsets and first requests: of its first half on this
+                    // path, else as the sub-steps below leave them
+                    prepare(r + 1, buf ^ 1);
+                    const bool next_sliced = tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1);
+                    sliced_request_half(buf ^ 1, 0, next_sliced);
+#pragma unroll
+                    for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j], !next_sliced);
+                }
+                if constexpr (kSlicedLocal) {
+                    // ---- stream (+) local operand in the bit-plane domain, half a tile at a time:
+                    //      four sub-steps turn the local values into deltas (as the general path
+                    //      does) and the deltas into two's-complement planes, a row of words per
+                    //      plane in LDS; then a lane takes a block: the incoming block's words from
+                    //      its registers, the local block's planes from the rows, sum, rate selection,
+                    //      payload words into the stage.
+                    uint32_t *rows = reinterpret_cast<uint32_t *>(s_in[wave]);
+                    bool fell_back = false;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        bool all4 = true;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int s = 4 * half + j;
+                            SubRegs<LOCAL> &L = loc[s % kDepth];
+                            int32_t v[8];
+                            local_deltas(L, v);
+                            {   // the freed registers go out for the sub-step kDepth further on (the next tile's at the end)
+                                const int wrap = s + kDepth >= kSub ? 1 : 0;
+                                request_local(r + wrap, s + kDepth - wrap * kSub, L);
+                            }
+                            // element 0 of a block stays out of the planes (its delta is the value itself)
+                            const uint32_t b0 = (uint32_t)v[0];
+                            if (k == 0) v[0] = 0;
+                            int32_t mx = v[0] > v[1] ? v[0] : v[1], mn = v[0] < v[1] ? v[0] : v[1];
+#pragma unroll
+                            for (int m = 2; m < 8; ++m) {
+                                mx = mx > v[m] ? mx : v[m];
+                                mn = mn < v[m] ? mn : v[m];
+                            }
+                            const int32_t z = mx > ~mn ? mx : ~mn;   // deltas within -(z + 1) .. z
+                            all4 = all4 && __builtin_amdgcn_ballot_w64(z > 7) == 0;
+                            const uint32_t at = (uint32_t)(j * 16 + quad);   // the block's lane in the second phase
+                            rows[(uint32_t)k * 64u + at] = local_planes4(v, sel1, sel2);   // plane k
+                            if (k == 0) rows[kLocalFew * 64u + at] = b0;
+                        }
+                        wave_lds_fence();
+                        SlicedIn A;
+                        sliced_take<kFewer>(sl_raw[0], sl_dig[0], A);
+                        if (half == 0) sliced_request_half(buf, 1, true);   // on its way while the first half is summed
+                        if (all4) {
+                            SlicedOut out;
+                            const uint32_t b0 = rows[kLocalFew * 64u + (uint32_t)lane];
+                            uint32_t plB[kLocalFew];
+#pragma unroll
+                            for (uint32_t q = 0; q < kLocalFew; ++q) plB[q] = rows[q * 64u + (uint32_t)lane];
+                            sliced_add_local<kFewer, kLocalFew>(A, plB, b0, out);
+                            wave_lds_fence();   // the rows are rewritten by the next half
+                            s_hdr_out[wave][half * 64 + lane] = (uint8_t)out.hdr;
+                            const uint32_t incl = wave_incl_scan_u32(out.size, lane);
+                            const uint32_t first32 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
+                            const uint32_t all64 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+                            // two writes of 32 blocks each, so that what is written at once fits an empty slot
+#pragma unroll
+                            for (int q = 0; q < 2; ++q) {
+                                const uint32_t bytes = q ? all64 - first32 : first32;
+                                make_room(bytes);   // always true here: 32 blocks fit an empty slot
+                                const uint32_t pos = run - flushed + (incl - out.size) - (q ? first32 : 0u);
+                                if ((lane >> 5) == q) sliced_write<kLocalFew + 1>((lds_bytes)stage, pos, out);
+                                run += bytes;
+                            }
+                        } else {
+                            // local deltas beyond the planes: these four sub-steps go down the general
+                            // path after all, their operands fetched again on the spot
+                            fell_back = true;
+#pragma unroll 1
+                            for (int s = 4 * half; s < 4 * half + 4; ++s) {
+                                SubRegs<LOCAL> again;
+                                InRegs again_in[kIn];
+                                request_local(r, s, again);
+                                request_in(0, r, buf, s, again_in);
+                                sub(s, again, again_in, r, buf, s, false);
+                            }
+                        }
+                    }
+                    wave_lds_fence();
+                    if (fell_back) sl_trust = false;
+                    prepare(r + 1, buf ^ 1);
+                    const bool next_sliced = tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1);
+                    sliced_request_half(buf ^ 1, 0, next_sliced);
+#pragma unroll
+                    for (int j = 0; j < kDepth; ++j) request_in(0, r + 1, buf ^ 1, j, in[j], !next_sliced);
+                }
+            } else {
+            planes_seen = 0;
 #pragma unroll 1
             for (int s = 0; s < kSub; s += kDepth) {
                 // the requests of the last kDepth sub-steps are the next tile's, whose block offsets
@@ -804,7 +929,8 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
                 for (int j = 0; j < kDepth; ++j) sub(s + j, loc[j], in[j], r + wrap, buf ^ wrap, s2 + j);
             }
-            if constexpr (kSliced) sliced_request_half(buf ^ 1, 0, tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1));
+            if constexpr (kSlicedLocal) sl_trust = __builtin_amdgcn_ballot_w64(planes_seen > kFewPlanes) == 0;
+            if constexpr (kAnySliced) sliced_request_half(buf ^ 1, 0, tile_of(r + 1) < n_tiles && sliced_ctx(buf ^ 1));
             }
             if constexpr (kEnc) {
                 wave_lds_fence();
@@ -1066,7 +1192,7 @@ __global__ void k_fill_u64(uint64_t *p, uint64_t n)
 
 // ---------------------------------------------------------------- launchers
 
-template <int NIN, int LOCAL, int OUT>
+template <int NIN, int LOCAL, int OUT, bool BITPLANE>
 static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     // data workgroups of four waves (one tile per wave and round), on the encoder + the scan server
@@ -1075,18 +1201,18 @@ static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_
     if (grid > max_grid) grid = max_grid;
     if (grid < 1u + extra) grid = 1u + extra;
     const uint32_t dyn = OUT == kOutStream ? (kWG / 64) * p.stage_bytes : 0u;
-    hipLaunchKernelGGL((k_wave<NIN, LOCAL, OUT>), dim3(grid), dim3(kWG), dyn, s, p);
+    hipLaunchKernelGGL((k_wave<NIN, LOCAL, OUT, BITPLANE>), dim3(grid), dim3(kWG), dyn, s, p);
     return hipGetLastError();
 }
 
-template <int NIN, int LOCAL, int OUT>
+template <int NIN, int LOCAL, int OUT, bool BITPLANE>
 static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
 {
     const size_t dyn = OUT == kOutStream ? (size_t)(kWG / 64) * stage_bytes : 0;
-    const void *fn = reinterpret_cast<const void *>(&k_wave<NIN, LOCAL, OUT>);
+    const void *fn = reinterpret_cast<const void *>(&k_wave<NIN, LOCAL, OUT, BITPLANE>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT>, kWG, dyn);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT, BITPLANE>, kWG, dyn);
     // The stream-producing kernels need every workgroup of the grid resident at the same time
     // (the scan's waits).  Near the LDS limit the runtime's answer was one workgroup too many on
     // MI355X (5 x 32 688 bytes reported to fit 160 KiB; the fifth was not resident and the waits
@@ -1104,14 +1230,25 @@ static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
     return e;
 }
 
+// both kinds of a kernel: the smaller of the two answers
+template <int NIN, int LOCAL, int OUT>
+static hipError_t both_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
+{
+    int with = 0, without = 0;
+    hipError_t e = wave_resident_blocks<NIN, LOCAL, OUT, true>(&with, stage_bytes);
+    if (e == hipSuccess) e = wave_resident_blocks<NIN, LOCAL, OUT, false>(&without, stage_bytes);
+    *blocks_per_cu = with < without ? with : without;
+    return e;
+}
+
 hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu)
 {
     switch (op) {
-    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
-    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32>(blocks_per_cu, stage_bytes);
-    case kOpHomSumF32: return wave_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
-    case kOpHomSumI32: return wave_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes);
-    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream, false>(blocks_per_cu, stage_bytes);
+    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32, false>(blocks_per_cu, stage_bytes);
+    case kOpHomSumF32: return both_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpHomSumI32: return both_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes);
+    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream, true>(blocks_per_cu, stage_bytes);
     default: return hipErrorInvalidValue;
     }
 }
@@ -1119,11 +1256,15 @@ hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu)
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     switch (op) {
-    case kOpCompress: return launch_wave<0, kLocalF32, kOutStream>(p, max_grid, s);
-    case kOpDecompress: return launch_wave<1, kLocalNone, kOutF32>(p, max_grid, s);
-    case kOpHomSumF32: return launch_wave<1, kLocalF32, kOutStream>(p, max_grid, s);
-    case kOpHomSumI32: return launch_wave<1, kLocalI32, kOutStream>(p, max_grid, s);
-    case kOpHomAdd: return launch_wave<2, kLocalNone, kOutStream>(p, max_grid, s);
+    case kOpCompress: return launch_wave<0, kLocalF32, kOutStream, false>(p, max_grid, s);
+    case kOpDecompress: return launch_wave<1, kLocalNone, kOutF32, false>(p, max_grid, s);
+    case kOpHomSumF32:
+        return p.sliced ? launch_wave<1, kLocalF32, kOutStream, true>(p, max_grid, s)
+                        : launch_wave<1, kLocalF32, kOutStream, false>(p, max_grid, s);
+    case kOpHomSumI32:
+        return p.sliced ? launch_wave<1, kLocalI32, kOutStream, true>(p, max_grid, s)
+                        : launch_wave<1, kLocalI32, kOutStream, false>(p, max_grid, s);
+    case kOpHomAdd: return launch_wave<2, kLocalNone, kOutStream, true>(p, max_grid, s);
     default: return hipErrorInvalidValue;
     }
 }
