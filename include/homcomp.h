@@ -99,6 +99,21 @@ int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEl
 int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
                            size_t nbEle, float eb, float *d_out, void *stream);
 
+/* GSZ_compress_deviceptr_plain / GSZ_decompress_deviceptr_plain (include/GSZ_entry.h:8-13,
+ * src/GSZ_entry.cu:150-228, kernels src/GSZ.cu:1475-1991): the plain codec, without the outlier
+ * mode.  A block's header byte is the bit width of its largest |delta| (capped at 31, as in the
+ * outlier codec), its payload the sign word and that many planes.  A plain stream is a stream
+ * of the outlier codec whose blocks are all in plain mode: homcomp_decompress_f32 and the
+ * homomorphic sums read it too.  The plain decoder has no out-of-bound rule (the reference's
+ * kernel never looks at cmpSize): the buffer must hold the whole stream.  The reference's
+ * wrapper reports a cmpSize that leaves out the payload of the last 32768-element chunk
+ * (src/GSZ_entry.cu:176-180 reads the exclusive offset of the last thread block); the length
+ * reported here is the true one. */
+int homcomp_compress_plain_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float eb,
+                               unsigned char *d_cmp, uint64_t *d_stream_len, void *stream);
+int homcomp_decompress_plain_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t nbEle, float eb,
+                                 float *d_out, void *stream);
+
 /* homomorphic_sum_F (include/GSZ_entry.h:33-36, src/GSZ_entry.cu:504-550): out = encode(
  * deltas(in) + Lorenzo(quantise(local))). */
 int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,

@@ -126,8 +126,10 @@ static int planes_of(uint32_t m)
     return b > 31 ? 31 : b;
 }
 
-/* src/GSZ.cu:86-164: sign map, absolute values, the two maxima, rate selection. */
-static void blk_analyse(const int32_t d[32], hco_blk *k)
+/* src/GSZ.cu:86-164: sign map, absolute values, the two maxima, rate selection.
+ * plain != 0: the plain codec of src/GSZ.cu:1475-1748, whose only rate is the bit width of the
+ * block maximum (:1578-1581) -- the first arm below, always. */
+static void blk_analyse(const int32_t d[32], hco_blk *k, int plain)
 {
     uint32_t max1 = 0, max2 = 0;
     k->sign = 0;
@@ -146,7 +148,7 @@ static void blk_analyse(const int32_t d[32], hco_blk *k)
     int ob = (hco_bit_num(k->a[0]) + 7) / 8;        /* :154 */
     uint32_t sz1 = fr1 ? 4u + 4u * (uint32_t)fr1 : 0u;   /* :156 */
     uint32_t sz2 = 4u + 4u * (uint32_t)fr2 + (uint32_t)ob; /* :157, both arms */
-    if (sz1 <= sz2) {                               /* :158-160 */
+    if (plain || sz1 <= sz2) {                      /* :158-160; plain codec: :1578-1581 */
         k->outlier_mode = 0;
         k->F = fr1;
         k->ob = 0;
@@ -209,7 +211,7 @@ uint32_t hco_block_size_from_header(uint8_t hdr)
 uint8_t hco_block_select(const int32_t delta[32], uint32_t *size)
 {
     hco_blk k;
-    blk_analyse(delta, &k);
+    blk_analyse(delta, &k, 0);
     if (size)
         *size = k.size;
     return k.hdr;
@@ -218,7 +220,16 @@ uint8_t hco_block_select(const int32_t delta[32], uint32_t *size)
 size_t hco_block_encode(const int32_t delta[32], uint8_t *out, uint8_t *hdr)
 {
     hco_blk k;
-    blk_analyse(delta, &k);
+    blk_analyse(delta, &k, 0);
+    if (hdr)
+        *hdr = k.hdr;
+    return blk_pack(&k, out);
+}
+
+size_t hco_block_encode_plain(const int32_t delta[32], uint8_t *out, uint8_t *hdr)
+{
+    hco_blk k;
+    blk_analyse(delta, &k, 1);
     if (hdr)
         *hdr = k.hdr;
     return blk_pack(&k, out);
@@ -278,6 +289,7 @@ typedef struct {
     size_t n;
     float recip;
     int n_in;            /* incoming streams to decode and add (0, 1 or 2)           */
+    int plain;           /* encode with the plain codec (no outlier mode)            */
     hco_instream in[2];
 } hco_src;
 
@@ -391,7 +403,7 @@ static int run_encode(const hco_src *s, size_t n, uint8_t *cmp, size_t *stream_l
             int32_t d[32];
             hco_blk k;
             produce_block(s, b, ofs, d);
-            blk_analyse(d, &k);
+            blk_analyse(d, &k, s->plain);
             cmp[b] = k.hdr;                         /* :167 */
             total += k.size;
         }
@@ -414,7 +426,7 @@ static int run_encode(const hco_src *s, size_t n, uint8_t *cmp, size_t *stream_l
             int32_t d[32];
             hco_blk k;
             produce_block(s, b, ofs, d);
-            blk_analyse(d, &k);
+            blk_analyse(d, &k, s->plain);
             if (block_ofs)
                 block_ofs[b] = o;
             o += blk_pack(&k, cmp + o);
@@ -471,6 +483,18 @@ int hco_compress(const float *x, size_t n, float eb, uint8_t *cmp, size_t *strea
     s.n = n;
     s.recip = recip_of(eb);
     return run_encode(&s, n, cmp, stream_len, block_ofs);
+}
+
+/* src/GSZ.cu:1475-1748 + src/GSZ_entry.cu:150-190: the plain codec. */
+int hco_compress_plain(const float *x, size_t n, float eb, uint8_t *cmp, size_t *stream_len)
+{
+    hco_src s;
+    memset(&s, 0, sizeof s);
+    s.x = x;
+    s.n = n;
+    s.recip = recip_of(eb);
+    s.plain = 1;
+    return run_encode(&s, n, cmp, stream_len, NULL);
 }
 
 int hco_encode_deltas(const int32_t *delta, size_t n, uint8_t *cmp, size_t *stream_len)
@@ -585,4 +609,67 @@ int hco_decode_deltas(const uint8_t *cmp, size_t cmp_size, size_t n, int32_t *de
 int hco_decode_quants(const uint8_t *cmp, size_t cmp_size, size_t n, int32_t *q)
 {
     return run_decode(cmp, cmp_size, n, 0.0f, 1, q);
+}
+
+/* src/GSZ.cu:1750-1991 + src/GSZ_entry.cu:192-228: the plain decoder.  A header byte is a plane
+ * count and nothing else (:1783-1784); offsets are the prefix sums of 4 + 4 * F per non-empty
+ * block (:1784, :1867-1880); there is no out-of-bound rule; a block is the sign word (:1887-1891)
+ * and F planes (:1897-1960), then the running sum and the dequantisation (:1963-1986).  Rate-0
+ * blocks come out as 0.0f (the reference leaves them unwritten). */
+int hco_decompress_plain(const uint8_t *cmp, size_t n, float eb, float *out)
+{
+    size_t nc = chunks_of(n);
+    if (nc == 0)
+        return 0;
+    uint64_t *excl = (uint64_t *)malloc((nc + 1) * sizeof(uint64_t));
+    if (!excl)
+        return -1;
+    HCO_PARALLEL_FOR
+    for (size_t c = 0; c < nc; c++) {
+        uint64_t total = 0;
+        for (size_t j = 0; j < BLOCKS_PER_CHUNK; j++) {
+            uint32_t F = cmp[c * BLOCKS_PER_CHUNK + j];
+            total += F ? 4u + 4u * F : 0u;
+        }
+        excl[c + 1] = total;
+    }
+    excl[0] = hco_header_bytes(n);
+    for (size_t c = 0; c < nc; c++)
+        excl[c + 1] += excl[c];
+    HCO_PARALLEL_FOR
+    for (size_t c = 0; c < nc; c++) {
+        uint64_t o = excl[c];
+        for (size_t j = 0; j < BLOCKS_PER_CHUNK; j++) {
+            size_t b = c * BLOCKS_PER_CHUNK + j;
+            uint32_t F = cmp[b];
+            uint32_t a[32];
+            uint32_t sign = 0;
+            memset(a, 0, sizeof a);
+            if (F) {
+                const uint8_t *in = cmp + o;
+                sign = ((uint32_t)in[0] << 24) | ((uint32_t)in[1] << 16) | ((uint32_t)in[2] << 8) | (uint32_t)in[3];
+                for (uint32_t p = 0; p < F; p++)
+                    for (int byte = 0; byte < 4; byte++) {
+                        uint32_t v = in[4 + 4 * p + (uint32_t)byte];
+                        for (int m = 0; m < 8; m++)
+                            if (p < 32)
+                                a[byte * 8 + m] |= ((v >> (7 - m)) & 1u) << p;
+                    }
+                o += 4u + 4u * F;
+            }
+            int32_t q = 0;
+            for (int i = 0; i < 32; i++) {
+                size_t e = b * HCO_BLOCK + (size_t)i;
+                uint32_t d = (sign >> (31 - i)) & 1u ? (uint32_t)0 - a[i] : a[i];
+                q = (int32_t)((uint32_t)q + d);
+                if (e >= n)
+                    break;
+                volatile float t = (float)q * eb;
+                volatile float v = t * 2.0f;
+                out[e] = v;
+            }
+        }
+    }
+    free(excl);
+    return 0;
 }

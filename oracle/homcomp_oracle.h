@@ -19,6 +19,9 @@
  *   stream scan         exclusive prefix sum vs numpy cumsum of the independent model's sizes.
  *   decompress          decode(encode)=id on ints, dequantisation closed form.
  *   hom sums            integer homomorphism q(A)+q(B), independent numpy model.
+ *   plain codec         the hand-derived blocks re-derived without the outlier arm; equals the
+ *                       outlier codec's stream wherever no block selects outlier mode and its
+ *                       plain arm block by block; independent numpy model; decode(encode)=id.
  * The reference holds no golden vectors and cannot be built here (CUDA + inline PTX, no nvcc),
  * so nothing is pinned by an execution of the reference itself.
  */
@@ -73,6 +76,14 @@ void hco_quantize_array(const float *x, size_t n, float eb, int32_t *q);
  * byte offset of every block's payload. Returns 0 on success. */
 int hco_compress(const float *x, size_t n, float eb, uint8_t *cmp, size_t *stream_len,
                  uint64_t *block_ofs);
+/* The plain codec (no outlier mode): src/GSZ.cu:1475-1748 (compress) and :1750-1991 (decompress),
+ * wrappers src/GSZ_entry.cu:150-228.  The header byte of a block is the bit width of its largest
+ * |delta|; the payload is the sign word and that many planes, or nothing for a zero block.  The
+ * reference's wrapper reports cmpOffset[gsize-1] + header bytes as cmpSize, which leaves out the
+ * payload of the last 32768-element chunk; *stream_len here is the true length. */
+int hco_compress_plain(const float *x, size_t n, float eb, uint8_t *cmp, size_t *stream_len);
+int hco_decompress_plain(const uint8_t *cmp, size_t n, float eb, float *out);
+size_t hco_block_encode_plain(const int32_t delta[32], uint8_t *out, uint8_t *hdr);
 /* Same back end fed with ready-made deltas (length n, zero padded). */
 int hco_encode_deltas(const int32_t *delta, size_t n, uint8_t *cmp, size_t *stream_len);
 

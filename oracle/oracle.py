@@ -63,6 +63,10 @@ def lib() -> C.CDLL:
         L.hco_quantize_array.argtypes = [f32p, C.c_size_t, C.c_float, i32p]
         L.hco_compress.argtypes = [f32p, C.c_size_t, C.c_float, u8p, szp, u64p]
         L.hco_encode_deltas.argtypes = [i32p, C.c_size_t, u8p, szp]
+        L.hco_compress_plain.argtypes = [f32p, C.c_size_t, C.c_float, u8p, szp]
+        L.hco_decompress_plain.argtypes = [u8p, C.c_size_t, C.c_float, f32p]
+        L.hco_block_encode_plain.argtypes = [i32p, u8p, u8p]
+        L.hco_block_encode_plain.restype = C.c_size_t
         L.hco_decompress.argtypes = [u8p, C.c_size_t, C.c_size_t, C.c_float, f32p]
         L.hco_decode_deltas.argtypes = [u8p, C.c_size_t, C.c_size_t, i32p]
         L.hco_decode_quants.argtypes = [u8p, C.c_size_t, C.c_size_t, i32p]
@@ -185,6 +189,34 @@ def compress(x, eb: float, want_offsets: bool = False):
     assert rc == 0
     out = cmp[:L.value].copy()
     return (out, ofs) if want_offsets else out
+
+
+def compress_plain(x, eb: float) -> np.ndarray:
+    """The plain codec's stream (true length)."""
+    x = _f32(x)
+    n = x.size
+    cmp = np.zeros(max_stream_bytes(n) + 4 * header_bytes(n), np.uint8)
+    L = C.c_size_t()
+    rc = lib().hco_compress_plain(_p(x, C.c_float), n, np.float32(eb), _p(cmp, C.c_uint8), C.byref(L))
+    assert rc == 0
+    return cmp[:L.value].copy()
+
+
+def decompress_plain(cmp, n: int, eb: float) -> np.ndarray:
+    buf = _padded_stream(cmp, n)
+    out = np.zeros(n, np.float32)
+    rc = lib().hco_decompress_plain(_p(buf, C.c_uint8), n, np.float32(eb), _p(out, C.c_float))
+    assert rc == 0
+    return out
+
+
+def block_encode_plain(delta) -> tuple[int, bytes]:
+    d = _i32(delta)
+    assert d.size == 32
+    out = np.zeros(160, np.uint8)
+    hdr = C.c_uint8()
+    n = lib().hco_block_encode_plain(_p(d, C.c_int32), _p(out, C.c_uint8), C.byref(hdr))
+    return int(hdr.value), out[:n].tobytes()
 
 
 def encode_deltas(delta) -> np.ndarray:

@@ -85,5 +85,27 @@ int main(int argc, char **argv)
         !write_bytes((prefix + ".dec").c_str(), h_dec.data(), n * 4))
         return 4;
     std::printf("n=%zu cmpSize=%zu sumSize=%zu sumSizeI=%zu header=%zu\n", n, cmpSize, sumSize, sumSizeI, hdr);
+
+    // the plain codec: device pointers, then the same through the host-pointer entries
+    size_t plainSize = 0, hostSize = 0;
+    GSZ_compress_deviceptr_plain(d_a, d_cmp, n, &plainSize, eb);
+    CHECK_HC();
+    GSZ_decompress_deviceptr_plain(d_dec, d_cmp, n, plainSize, eb);
+    CHECK_HC();
+    std::vector<unsigned char> h_plain(plainSize), h_host(cap);
+    std::vector<float> h_pdec(n), h_hdec(n, -1.0f);
+    CHECK_HIP(hipMemcpy(h_plain.data(), d_cmp, plainSize, hipMemcpyDeviceToHost));
+    CHECK_HIP(hipMemcpy(h_pdec.data(), d_dec, n * 4, hipMemcpyDeviceToHost));
+    std::vector<float> a_copy(a);
+    GSZ_compress_hostptr(a_copy.data(), h_host.data(), n, &hostSize, eb);
+    CHECK_HC();
+    GSZ_decompress_hostptr(h_hdec.data(), h_host.data(), n, hostSize, eb);
+    CHECK_HC();
+    if (!write_bytes((prefix + ".plain").c_str(), h_plain.data(), plainSize) ||
+        !write_bytes((prefix + ".plain_host").c_str(), h_host.data(), hostSize) ||
+        !write_bytes((prefix + ".plain_dec").c_str(), h_pdec.data(), n * 4) ||
+        !write_bytes((prefix + ".plain_host_dec").c_str(), h_hdec.data(), n * 4))
+        return 4;
+    std::printf("plainSize=%zu hostSize=%zu\n", plainSize, hostSize);
     return 0;
 }

@@ -42,28 +42,29 @@ def lorenzo(q: np.ndarray) -> np.ndarray:
     return D.reshape(-1)[: n + pad].astype(np.int32)
 
 
-def select(D: np.ndarray):
-    """D: (blocks, 32) int64 deltas -> header bytes, payload sizes, (outlier, F, ob)."""
+def select(D: np.ndarray, plain: bool = False):
+    """D: (blocks, 32) int64 deltas -> header bytes, payload sizes, (outlier, F, ob).
+    plain: the plain codec (HomComp/src/GSZ.cu:1578-1581), which has no outlier mode."""
     A = np.abs(D)
     fr1 = np.minimum(bit_length(A.max(axis=1)), 31)
     fr2 = np.minimum(bit_length(A[:, 1:].max(axis=1)), 31)
     ob = (bit_length(A[:, 0]) + 7) // 8
     sz1 = np.where(fr1 > 0, 4 + 4 * fr1, 0)
     sz2 = 4 + 4 * fr2 + ob
-    outl = sz1 > sz2
+    outl = (sz1 > sz2) & (not plain)
     hdr = np.where(outl, fr2 | 0x80 | ((ob - 1) << 5), fr1).astype(np.uint8)
     size = np.where(outl, sz2, sz1)
     return hdr, size, outl, np.where(outl, fr2, fr1), np.where(outl, ob, 0)
 
 
-def encode_deltas(d: np.ndarray):
+def encode_deltas(d: np.ndarray, plain: bool = False):
     """Returns (stream, block_offsets)."""
     n = d.size
     npad = (n + CHUNK - 1) // CHUNK * CHUNK
     D = np.zeros(npad, np.int64)
     D[:n] = d
     D = D.reshape(-1, 32)
-    hdr, size, outl, F, ob = select(D)
+    hdr, size, outl, F, ob = select(D, plain)
     ofs = hdr.size + np.concatenate([[0], np.cumsum(size)])
     out = np.zeros(int(ofs[-1]), np.uint8)
     out[: hdr.size] = hdr
@@ -85,12 +86,12 @@ def encode_deltas(d: np.ndarray):
     return out, ofs
 
 
-def compress(x: np.ndarray, eb):
+def compress(x: np.ndarray, eb, plain: bool = False):
     n = x.size
     npad = (n + CHUNK - 1) // CHUNK * CHUNK
     xp = np.zeros(npad, np.float32)
     xp[:n] = x
-    return encode_deltas(lorenzo(quantize(xp, eb)))
+    return encode_deltas(lorenzo(quantize(xp, eb)), plain)
 
 
 def decode_deltas(stream: np.ndarray, n: int) -> np.ndarray:

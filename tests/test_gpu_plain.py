@@ -1,0 +1,106 @@
+"""The plain codec (HomComp/src/GSZ.cu:1475-1991, no outlier mode) through the C ABI against the
+CPU oracle: byte-exact streams, bit-exact decompressed values, and the relations that tie it to
+the outlier codec (a plain stream is a stream of the outlier codec whose blocks are all in plain
+mode, so the outlier decoder and the homomorphic sums read it too)."""
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, first_diff
+
+pytestmark = pytest.mark.gpu
+
+MAX_N = 1 << 22
+
+
+@pytest.fixture(scope="module")
+def gpu(pkg, cuda):
+    g = Gpu(pkg, cuda, MAX_N)
+    yield g
+    g.close()
+
+
+def gpu_compress_plain(g, x, eb, offset=0):
+    dx = g.dev(x)
+    cmp = g.stream_buf(x.size, offset=offset)
+    dlen = g.torch.zeros(1, dtype=g.torch.int64, device="cuda")
+    g.ws.compress_plain(dx, float(eb), cmp, stream_len=dlen, n=x.size)
+    L = g.ws.last_size()
+    assert int(dlen.item()) == L
+    return cmp[:L].cpu().numpy()
+
+
+def gpu_decompress_plain(g, s, n, eb, offset=0):
+    buf = g.put_stream(s, n, offset=offset)
+    out = g.torch.full((max(n, 1),), 7.0, dtype=g.torch.float32, device="cuda")
+    g.ws.decompress_plain(buf, n, float(eb), out)
+    g.torch.cuda.synchronize()
+    return out[:n].cpu().numpy()
+
+
+CASES = [("smooth", 1 << 20, 1e-4), ("smooth", 1 << 18, 1e-2), ("gradient_like", 1 << 19, 1e-6),
+         ("gradient_like", 1 << 19, 1e-2), ("uniform", 1 << 19, 1e-4), ("uniform", (1 << 16) + 13, 1e-6),
+         ("smooth", 32768 + 1, 1e-4), ("uniform", 33, 1e-3), ("smooth", (1 << 22) - 4099, 1e-3)]
+
+
+@pytest.mark.parametrize("kind,n,rel", CASES)
+def test_plain_codec(gpu, orc, gen, kind, n, rel):
+    orc.set_threads(16)
+    x = gen.GENERATORS_NP[kind](n, 3)
+    mn, mx = orc.value_range(x)
+    eb = orc.rel_to_abs(rel, mn, mx)
+    want = orc.compress_plain(x, eb)
+    got = gpu_compress_plain(gpu, x, eb)
+    assert got.size == want.size and np.array_equal(got, want), first_diff(got, want)
+    hb = orc.header_bytes(n)
+    assert not (got[:hb] >= 32).any(), "a plain header byte is a plane count"
+    want_dec = orc.decompress_plain(want, n, eb)
+    dec = gpu_decompress_plain(gpu, want, n, eb)
+    assert np.array_equal(dec.view(np.uint32), want_dec.view(np.uint32))
+    # the outlier decoder reads the plain stream to the same values, and they are the values of
+    # the outlier codec's own stream
+    dec2 = gpu.decompress(want, n, eb)
+    assert np.array_equal(dec2.view(np.uint32), want_dec.view(np.uint32))
+    assert np.array_equal(want_dec.view(np.uint32), orc.decompress(orc.compress(x, eb), n, eb).view(np.uint32))
+    err = np.abs(dec.astype(np.float64) - x.astype(np.float64))
+    assert (err <= float(eb) + 2.0 ** -21 * np.abs(x.astype(np.float64))).all()
+
+
+def test_plain_equals_outlier_codec_without_outlier_blocks(gpu, orc, gen):
+    """White noise at a coarse bound puts no block into outlier mode: both codecs, one stream."""
+    n = 1 << 18
+    x = gen.uniform_np(n, 8)
+    eb = np.float32(1e-3)
+    so = gpu.compress(x, eb)
+    assert not (so[:orc.header_bytes(n)] >= 128).any()
+    assert np.array_equal(gpu_compress_plain(gpu, x, eb), so)
+
+
+def test_plain_stream_into_a_homomorphic_sum(gpu, orc, gen):
+    """A plain stream as the incoming operand of hom_sum_f32 and hom_add (the result is re-encoded
+    by the outlier codec): the oracle's bytes, the integer sum of the quantised values."""
+    n = (1 << 18) + 4099
+    a, b = gen.smooth_np(n, 11), gen.smooth_np(n, 12)
+    eb = np.float32(8e-4)
+    sp = orc.compress_plain(a, eb)
+    want = orc.hom_sum_f32(sp, b, eb)
+    got = gpu.hom_sum_f32(sp, b, eb)
+    assert np.array_equal(got, want), first_diff(got, want)
+    assert np.array_equal(want, orc.hom_sum_f32(orc.compress(a, eb), b, eb))
+    got2 = gpu.hom_add(sp, orc.compress_plain(b, eb), n)
+    assert np.array_equal(got2, want), first_diff(got2, want)
+    assert np.array_equal(orc.decode_quants(got, n), orc.quantize_array(a, eb) + orc.quantize_array(b, eb))
+
+
+def test_plain_unaligned_and_saturated(gpu, orc):
+    rng = np.random.default_rng(5)
+    n = 1 << 15
+    x = rng.standard_normal(n).astype(np.float32)
+    x[5], x[77], x[1000] = np.nan, np.inf, -np.inf      # outside the codec's domain: plane counts stay capped at 31
+    x[::97] = 3e9
+    eb = np.float32(1e-3)
+    want = orc.compress_plain(x, eb)
+    for offset in (0, 3):
+        got = gpu_compress_plain(gpu, x, eb, offset=offset)
+        assert np.array_equal(got, want), first_diff(got, want)
+        dec = gpu_decompress_plain(gpu, want, n, eb, offset=offset)
+        assert np.array_equal(dec.view(np.uint32), orc.decompress_plain(want, n, eb).view(np.uint32))

@@ -39,3 +39,12 @@ def test_shim_roundtrip(tmp_path, orc, gen, cuda, n):
         assert np.array_equal(got_i, want_sum)
     dec = np.fromfile(str(prefix) + ".dec", np.float32)
     assert np.array_equal(dec.view(np.uint32), orc.decompress(want_sum, n, eb).view(np.uint32))
+    # the plain codec through the device-pointer and the host-pointer entries: true lengths
+    want_plain = orc.compress_plain(a, eb)
+    assert int(fields["plainSize"]) == want_plain.size and int(fields["hostSize"]) == want_plain.size
+    assert np.array_equal(np.fromfile(str(prefix) + ".plain", np.uint8), want_plain)
+    assert np.array_equal(np.fromfile(str(prefix) + ".plain_host", np.uint8), want_plain)
+    want_pdec = orc.decompress_plain(want_plain, n, eb)
+    for name in (".plain_dec", ".plain_host_dec"):
+        got = np.fromfile(str(prefix) + name, np.float32)
+        assert np.array_equal(got.view(np.uint32), want_pdec.view(np.uint32)), name

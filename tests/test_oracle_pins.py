@@ -106,6 +106,56 @@ def test_handbuilt_block_vectors(orc, vec):
     assert s[0] == vec["header"] and list(s[1024:]) == vec["payload"]
 
 
+@pytest.mark.parametrize("vec", load_vectors(), ids=lambda v: v["name"].split(":")[0])
+def test_handbuilt_block_vectors_plain_codec(orc, vec):
+    """The same blocks under the plain codec (HomComp/src/GSZ.cu:1475-1748): header = bit width of
+    the largest |delta|, payload = sign word + planes with element 0 left in place."""
+    d = np.zeros(32, np.int32)
+    for i, v in enumerate(vec.get("delta", [])):
+        d[i] = v
+    for i, v in vec.get("sparse", {}).items():
+        d[int(i)] = v
+    hdr, payload = orc.block_encode_plain(d)
+    assert hdr == vec["plain_header"]
+    assert list(payload) == vec["plain_payload"]
+    # a plain block is a plain-mode block of the outlier codec: its decoder reads it back
+    assert np.array_equal(orc.block_decode(hdr, payload), d)
+    s, _ = M.encode_deltas(d, plain=True)
+    assert s[0] == vec["plain_header"] and list(s[1024:]) == vec["plain_payload"]
+    # where the outlier codec chooses its plain arm the two codecs agree
+    if vec["header"] < 128:
+        assert (hdr, list(payload)) == (vec["header"], vec["payload"])
+
+
+def test_plain_codec_streams(orc, gen):
+    """Plain streams against the independent model and against the outlier codec: identical
+    wherever no block selects outlier mode, never shorter in header count, decode(encode) = id
+    through both decoders, error bound."""
+    rng = np.random.default_rng(41)
+    for n, maker, eb in ((32768, gen.uniform_np, 1e-3), (50000, gen.smooth_np, 2e-4), (40000, gen.gradient_like_np, 1e-6),
+                         (65536 + 77, gen.uniform_np, 1e-1)):
+        x = maker(n, int(rng.integers(1, 1000)))
+        eb = np.float32(eb)
+        sp = orc.compress_plain(x, eb)
+        want, _ = M.compress(x, eb, plain=True)
+        assert np.array_equal(sp, want), n
+        so = orc.compress(x, eb)
+        hb = orc.header_bytes(n)
+        if not (so[:hb] >= 128).any():
+            assert np.array_equal(sp, so)           # no block in outlier mode: the same stream
+        else:
+            assert sp.size >= so.size               # outlier mode is only ever chosen when it is shorter
+        # both decoders read a plain stream the same way, and give back the quantised values
+        dec = orc.decompress_plain(sp, n, eb)
+        assert np.array_equal(dec.view(np.uint32), orc.decompress(sp, n, eb).view(np.uint32))
+        assert np.array_equal(dec.view(np.uint32), orc.decompress(so, n, eb).view(np.uint32))
+        assert np.array_equal(orc.decode_quants(sp, n), orc.quantize_array(x, eb))
+        assert (np.abs(dec.astype(np.float64) - x) <= float(eb) + 2.0 ** -21 * np.abs(x)).all()
+    # uniform noise at a coarse bound has no outlier-mode blocks at all: exercised above?
+    x = gen.uniform_np(32768, 5)
+    assert not (orc.compress(x, np.float32(1e-3))[:1024] >= 128).any()
+
+
 def test_single_bit_positions(orc):
     """One set bit at element i, plane p lands at byte 4 + 4p + i/8, bit 7 - i%8 (plain mode)."""
     for i in range(1, 32):

@@ -19,6 +19,7 @@ EXPORTS = (
     "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
     "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
     "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_compress_f32", "homcomp_decompress_f32",
+    "homcomp_compress_plain_f32", "homcomp_decompress_plain_f32",
     "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add", "homcomp_hom_sum_f32_static",
     "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
 )
@@ -66,6 +67,8 @@ def lib() -> C.CDLL:
         L.homcomp_workspace_set_option.argtypes = [vp, C.c_int, C.c_long]
         L.homcomp_compress_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_decompress_f32.argtypes = [vp, vp, sz, sz, C.c_float, vp, vp]
+        L.homcomp_compress_plain_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
+        L.homcomp_decompress_plain_f32.argtypes = [vp, vp, sz, C.c_float, vp, vp]
         L.homcomp_hom_sum_f32.argtypes = [vp, vp, sz, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_hom_sum_i32.argtypes = [vp, vp, sz, vp, sz, vp, u64p, vp]
         L.homcomp_hom_add.argtypes = [vp, vp, sz, vp, sz, sz, vp, u64p, vp]
@@ -148,6 +151,16 @@ class Workspace:
         _check(lib().homcomp_compress_f32(self._h, data.data_ptr(), n, eb, cmp.data_ptr(),
                                           stream_len.data_ptr() if stream_len is not None else None,
                                           _stream_ptr(stream)), "compress_f32")
+
+    def compress_plain(self, data, eb: float, cmp, stream_len=None, n: int | None = None, stream=None):
+        n = data.numel() if n is None else n
+        _check(lib().homcomp_compress_plain_f32(self._h, data.data_ptr(), n, eb, cmp.data_ptr(),
+                                                stream_len.data_ptr() if stream_len is not None else None,
+                                                _stream_ptr(stream)), "compress_plain_f32")
+
+    def decompress_plain(self, cmp, n: int, eb: float, out, stream=None):
+        _check(lib().homcomp_decompress_plain_f32(self._h, cmp.data_ptr(), n, eb, out.data_ptr(),
+                                                  _stream_ptr(stream)), "decompress_plain_f32")
 
     def decompress(self, cmp, cmp_size: int, n: int, eb: float, out, stream=None):
         _check(lib().homcomp_decompress_f32(self._h, cmp.data_ptr(), cmp_size, n, eb,

@@ -565,6 +565,36 @@ int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEl
     return run_tile_op(ws, hc::kOpCompress, p, 0, s);
 }
 
+int homcomp_compress_plain_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float eb,
+                               unsigned char *d_cmp, uint64_t *d_stream_len, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_ws(ws, nbEle);
+    if (rc) return rc;
+    if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
+    if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
+    if (!d_data || !d_cmp) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_data)) return HOMCOMP_ERR_ALIGNMENT;
+    hc::TileParams p;
+    if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
+    p.local = d_data;
+    p.out_cmp = d_cmp;
+    p.eb = eb;
+    p.recip = 0.5f / eb;
+    p.user_total = d_stream_len;
+    p.plain = 1;
+    return run_tile_op(ws, hc::kOpCompress, p, 0, s);
+}
+
+int homcomp_decompress_plain_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t nbEle, float eb,
+                                 float *d_out, void *stream)
+{
+    // A plain stream is a stream of the outlier codec in which every block is in plain mode, so
+    // the one decoder reads both.  The plain decoder of the reference knows no stated size:
+    // every block is read.
+    return homcomp_decompress_f32(ws, d_cmp, homcomp_max_stream_bytes(nbEle), nbEle, eb, d_out, stream);
+}
+
 int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, size_t cmp_size,
                            size_t nbEle, float eb, float *d_out, void *stream)
 {

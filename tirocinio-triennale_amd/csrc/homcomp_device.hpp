@@ -194,8 +194,9 @@ __device__ __forceinline__ uint32_t transpose4(uint32_t y)
 // magnitudes, block-wide bit widths through the quad, rate selection.  `k` is the lane's
 // position in its quad.  hdr, size and a0 (|delta| of the block's element 0) come out identical
 // in the four lanes of a quad.
+// plain_only: the plain codec (HomComp/src/GSZ.cu:1578-1581), which knows no outlier mode.
 __device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8], uint32_t &sb,
-                                         uint32_t &hdr, uint32_t &size, uint32_t &a0)
+                                         uint32_t &hdr, uint32_t &size, uint32_t &a0, bool plain_only = false)
 {
     sb = 0;
     uint32_t rest = 0;
@@ -216,7 +217,7 @@ __device__ __forceinline__ void analyse8(const int32_t v[8], int k, uint32_t a[8
     uint32_t ob = (bit_num(a0) + 7u) >> 3;
     uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;              // :156
     uint32_t sz2 = 4u + 4u * fr2 + ob;                    // :157
-    if (sz1 <= sz2) {                                     // :158-160
+    if (plain_only || sz1 <= sz2) {                       // :158-160
         hdr = fr1;
         size = sz1;
     } else {                                              // :161-164

@@ -771,7 +771,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     //      sizes are equal in the four lanes of a quad, so a scan over the quads
                     //      minus the own size is the exclusive prefix in every lane
                     uint32_t a[8], sb, hd, size, a0;
-                    analyse8(v, k, a, sb, hd, size, a0);
+                    analyse8(v, k, a, sb, hd, size, a0, NIN == 0 && p.plain != 0);
                     const uint32_t incl = quad_incl_scan_u32(size);
                     const uint32_t sub_total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
                     if (k == 0) s_hdr_out[wave][s * 16 + quad] = (uint8_t)hd;
