@@ -487,6 +487,12 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     };
     // (`wanted` false: nothing is read, the registers are only given a value)
     auto request_in = [&](int c, int64_t r, int b, int s, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
+        if constexpr (kSliced) {
+            if (!wanted) {   // wave-uniform; cheaper here than a request that fetches nothing
+                in[c].chunk = u32x4{0u, 0u, 0u, 0u};
+                return;
+            }
+        }
         uintptr_t ga;
         uint32_t shift, nbytes, rel0;
         range_of(c, b, s, ga, shift, nbytes, rel0);
