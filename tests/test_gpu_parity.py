@@ -479,6 +479,35 @@ def test_lds_budget_follows_the_data(pkg, cuda, orc, gen):
         g.close()
 
 
+@pytest.mark.parametrize("forced", [None, "0", "2"])
+def test_sum_kernel_follows_the_incoming_tiles(pkg, cuda, orc, gen, monkeypatch, forced):
+    """stream (+) local operand comes as two kernels, with and without the bit-plane path; a
+    workspace picks by the incoming stream's size on its first call of a length and by the count
+    of tiles with few planes that the previous call of that length left behind afterwards
+    (HOMCOMP_SLICED forces one).  Sparse spikes over small values compress like few-plane data
+    although almost every tile holds a wide block, smooth data really is few-plane data: runs of
+    either, and changes between them on one workspace, must keep producing the oracle's bytes."""
+    if forced is not None:
+        monkeypatch.setenv("HOMCOMP_SLICED", forced)
+    orc.set_threads(16)
+    n = (1 << 21) + 4096 * 5 + 77
+    spiky = (gen.gradient_like_np(n, 61), gen.gradient_like_np(n, 62), np.float32(2e-2))
+    smooth = (gen.smooth_np(n, 63), gen.smooth_np(n, 64), np.float32(8e-4))
+    g = Gpu(pkg, cuda, n)
+    try:
+        want = {}
+        for name, (a, b, eb) in (("spiky", spiky), ("smooth", smooth)):
+            sa = orc.compress(a, eb)
+            qp = orc.quant_predict(b, eb)
+            want[name] = (sa, b, eb, qp, orc.hom_sum_f32(sa, b, eb), orc.hom_sum_i32(sa, qp))
+        for step, name in enumerate(["spiky", "spiky", "spiky", "smooth", "smooth", "spiky", "smooth", "smooth"]):
+            sa, b, eb, qp, want_f, want_i = want[name]
+            assert_stream_equal(g.hom_sum_f32(sa, b, eb), want_f, f"hom_sum_f32, call {step} ({name})")
+            assert_stream_equal(g.hom_sum_i32(sa, qp), want_i, f"hom_sum_i32, call {step} ({name})")
+    finally:
+        g.close()
+
+
 def test_two_streams_do_not_overlap_their_scans(pkg, cuda, orc, gen):
     """Two workspaces driven from two streams at the same time.  Every stream-producing kernel
     needs its whole grid resident, so the library orders such launches across the streams of a

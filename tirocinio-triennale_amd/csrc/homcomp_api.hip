@@ -60,10 +60,13 @@ struct homcomp_workspace {
     uint32_t max_grid[hc::kOpCount][3];  // persistent grid of each operation's kernel, per LDS budget (small, medium, large)
     uint32_t full_grid[hc::kOpCount][3]; // the same at 100 percent (HOMCOMP_OPT_GRID_PERCENT scales it)
     uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
+    uint64_t *h_few;          // pinned host word, left by the offsets pre-pass of the last stream (+) local operand call that
+                              // got that far: n_tiles << 32 | tiles none of whose blocks has more than three planes
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint32_t out_slots;       // deferral depth of packed tiles (2..4); the device's spill area has this many slots per data wave
     bool holds_spill;         // counted among the users of the device's spill area
-    uint32_t sliced;          // HOMCOMP_SLICED=0 switches the bit-plane path of stream (+) stream off
+    uint32_t sliced;          // bit-plane paths of the sums: HOMCOMP_SLICED=0 switches them off, 2 makes stream (+) local
+                              // operand take its own for every tile that allows it (1: where most tiles do)
     int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
 };
 
@@ -108,7 +111,7 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
 
 // Offsets pre-pass of the incoming streams (header bytes -> payload offset of every tile): one
 // pass of launches for all of them.
-int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s)
+int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s, bool report_few = false)
 {
     hc::InOffsetsArgs a;
     std::memset(&a, 0, sizeof a);
@@ -119,6 +122,7 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
         a.block_sums[c] = ws->d_in_blocks[c];
         a.ofs[c] = ws->d_in_ofs[c];
     }
+    if (report_few) a.few_report[0] = ws->h_few;
     return hip_ok(hc::launch_in_offsets(a, n_streams, p->n_tiles, p->hdr_bytes, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
@@ -266,9 +270,19 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         p.stage_bytes = 0u;
         return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
-    // stream (+) local operand: the kernel with the bit-plane path where the incoming blocks can
-    // have the few planes it takes (at most 4 + 4 * 3 + 4 bytes each on average), else the one without
-    if ((op == hc::kOpHomSumF32 || op == hc::kOpHomSumI32) && expected_tile_bytes > kBitplaneTileBytes) p.sliced = 0;
+    // stream (+) local operand: the kernel with the bit-plane path where most incoming tiles can
+    // take it, else the one without.  The offsets pre-pass counts the tiles of few planes and
+    // leaves the count in host-visible memory; it arrives too late for the launch it belongs to,
+    // so the choice follows the previous call of the same length (a ring step sums chunk after
+    // chunk of similar data), and the incoming stream's size where there is none (blocks of at
+    // most three planes are at most 4 + 4 * 3 + 4 bytes).  Either kernel produces the same bytes.
+    if ((op == hc::kOpHomSumF32 || op == hc::kOpHomSumI32) && p.sliced == 1u) {
+        const uint64_t seen = *(volatile const uint64_t *)ws->h_few;
+        if (seen >> 32 == p.n_tiles)
+            p.sliced = (seen & 0xffffffffu) * 4u >= (uint64_t)p.n_tiles * 3u;
+        else
+            p.sliced = expected_tile_bytes <= kBitplaneTileBytes;
+    }
     if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
     int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
     if (ws->stage_class >= 0) cls = ws->stage_class;
@@ -474,7 +488,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (std::strcmp(e, "large") == 0) ws->stage_class = 2;
     }
     ws->sliced = 1;
-    if (const char *e = std::getenv("HOMCOMP_SLICED")) ws->sliced = std::strtol(e, nullptr, 10) != 0;
+    if (const char *e = std::getenv("HOMCOMP_SLICED")) {
+        const long v = std::strtol(e, nullptr, 10);
+        ws->sliced = v < 0 ? 0 : (v > 2 ? 2 : (int)v);
+    }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {
         const long v = std::strtol(e, nullptr, 10);
@@ -486,14 +503,15 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (v >= 0 && v <= (long)kMaxEpoch) ws->epoch = (uint32_t)v;
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
-        !hip_ok(hipHostMalloc((void **)&ws->h_total, (2 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
+        !hip_ok(hipHostMalloc((void **)&ws->h_total, (3 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
         (void)spill_release(ws);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
-    std::memset(ws->h_total, 0, (2 + hc::kOpCount) * sizeof(uint64_t));
+    std::memset(ws->h_total, 0, (3 + hc::kOpCount) * sizeof(uint64_t));
     ws->h_mean_tile = ws->h_total + 2;
+    ws->h_few = ws->h_mean_tile + hc::kOpCount;
     uint8_t *base = (uint8_t *)ws->d_block;
     ws->d_tile_totals = (uint64_t *)(base + o_status);
     ws->d_tile_prefixes = ws->d_tile_totals + t;
@@ -636,7 +654,7 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s, true))) return rc;
     return run_tile_op(ws, hc::kOpHomSumF32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
@@ -657,7 +675,7 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.local = d_local_delta;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s, true))) return rc;
     return run_tile_op(ws, hc::kOpHomSumI32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 

@@ -337,8 +337,9 @@ struct InRegs {
 };
 
 // BITPLANE: the kernel has the bit-plane paths.  stream (+) local operand comes in both kinds: the
-// host launches the kind without them where the incoming stream is too wide for them anyway,
-// because the general path alone is the faster code for such data (fewer registers in use).
+// host launches the kind without them where the incoming streams are too wide for them anyway,
+// because the general path alone is the faster code for such data (fewer registers in use; a
+// tile of the general path costs about 8 % more in the kernel that has both).
 template <int NIN, int LOCAL, int OUT, bool BITPLANE>
 __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k_wave(const TileParams p)
 {
@@ -977,6 +978,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 // (`base` = header length).
 
 constexpr uint32_t kOfsBlockTiles = 256;
+constexpr uint32_t kBlockSumBits = 23;
 
 __device__ __forceinline__ uint32_t wg_reduce_u32(uint32_t v, uint32_t *s_tmp)
 {
@@ -1005,7 +1007,7 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
     uint64_t *__restrict__ ofs = direct ? a.ofs[blockIdx.y] : nullptr;
     __shared__ uint32_t s_tmp[4];
     __shared__ uint32_t s_tot[kOfsBlockTiles];
-    uint32_t acc = 0;
+    uint32_t acc = 0, few_tiles = 0;
     constexpr uint32_t kPieces = kTileBlocks / 16;            // 16-byte header pieces (lanes) per tile
     constexpr uint32_t kPasses = kOfsBlockTiles * kPieces / 256;
     // all pieces of the thread are requested before the first is used: the kernel is a handful of
@@ -1044,13 +1046,27 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
         sum += dpp_u32<kDppXor1>(sum);
         sum += dpp_u32<kDppXor2>(sum);
         sum += dpp_u32<kDppRowHalfMirror>(sum);   // the other quad of the eight
+        // plane counts of the tile's blocks, or-ed: at most kFewPlanes if every one of them is
+        uint32_t planes = (q[it].x | q[it].y | q[it].z | q[it].w) & 0x1f1f1f1fu;
+        planes |= planes >> 16;
+        planes = (planes | (planes >> 8)) & 0x1fu;
+        planes |= dpp_u32<kDppXor1>(planes);
+        planes |= dpp_u32<kDppXor2>(planes);
+        planes |= dpp_u32<kDppRowHalfMirror>(planes);
         if ((threadIdx.x & (kPieces - 1)) == 0) {
-            if (tile < n_tiles) totals[tile] = sum;
+            if (tile < n_tiles) {
+                totals[tile] = sum;
+                few_tiles += planes <= kFewPlanes ? 1u : 0u;
+            }
             s_tot[tile % kOfsBlockTiles] = sum;   // 0 beyond the last tile
         }
     }
     const uint32_t block_total = wg_reduce_u32(acc, s_tmp);   // with a barrier: s_tot is complete
-    if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total;
+    const uint32_t block_few = wg_reduce_u32(few_tiles, s_tmp);
+    // a block's bytes stay below 2^23 (256 tiles of at most 128 * 132 bytes): its count of tiles
+    // with few planes (at most 256) travels in the bits above
+    static_assert(kOfsBlockTiles * kTileBlocks * kMaxBlockBytes < (1u << kBlockSumBits), "packing of the block sums");
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total | (block_few << kBlockSumBits);
     if (ofs == nullptr) return;
     // one block of tiles: its offsets right away, as k_in_offsets below would compute them
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1063,7 +1079,10 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
     for (int q = 0; q < 4; ++q)
         if (q < wave) earlier += s_tmp[q];
     if (threadIdx.x < n_tiles) ofs[threadIdx.x] = base + earlier + (incl - mine);
-    if (threadIdx.x == 0) ofs[n_tiles] = base + block_total;   // the end of the payload
+    if (threadIdx.x == 0) {
+        ofs[n_tiles] = base + block_total;   // the end of the payload
+        if (a.few_report[blockIdx.y]) *a.few_report[blockIdx.y] = ((uint64_t)n_tiles << 32) | block_few;
+    }
 }
 
 __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base)
@@ -1075,11 +1094,15 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
     __shared__ uint32_t s_wave[4];
     // bytes of all earlier blocks (a block is at most 256 * 132 * 128 bytes, so 64-bit sums)
     uint64_t before = 0;
-    for (uint32_t q0 = 0; q0 < blockIdx.x; q0 += 256) {
+    uint32_t few_before = 0;
+    const bool last = (blockIdx.x + 1) * kOfsBlockTiles >= n_tiles;   // this block also reports the count of tiles with few planes
+    for (uint32_t q0 = 0; q0 < blockIdx.x + (last ? 1u : 0u); q0 += 256) {
         const uint32_t q = q0 + threadIdx.x;
-        const uint32_t v = q < blockIdx.x ? block_sums[q] : 0u;
+        const uint32_t packed = q <= blockIdx.x ? block_sums[q] : 0u;
+        const uint32_t v = q < blockIdx.x ? packed & ((1u << kBlockSumBits) - 1u) : 0u;
         // split so that the 32-bit reduction cannot overflow (256 values below 2^23 each)
         before += (uint64_t)wg_reduce_u32(v & 0xffffu, s_tmp) + ((uint64_t)wg_reduce_u32(v >> 16, s_tmp) << 16);
+        if (last) few_before += wg_reduce_u32(packed >> kBlockSumBits, s_tmp);   // its own block included
     }
     const uint32_t tile = blockIdx.x * kOfsBlockTiles + threadIdx.x;
     const uint32_t mine = tile < n_tiles ? totals[tile] : 0u;
@@ -1096,7 +1119,10 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
     }
     if (tile < n_tiles) ofs[tile] = base + before + earlier + (incl - mine);
     // the entry after the last tile is the end of the payload
-    if (threadIdx.x == 0 && (blockIdx.x + 1) * kOfsBlockTiles >= n_tiles) ofs[n_tiles] = base + before + block_total;
+    if (threadIdx.x == 0 && last) {
+        ofs[n_tiles] = base + before + block_total;
+        if (a.few_report[blockIdx.y]) *a.few_report[blockIdx.y] = ((uint64_t)n_tiles << 32) | few_before;
+    }
 }
 
 // HomComp/src/homcomp.cu:1553-1602: Lorenzo deltas of the quantised values as int32.

@@ -57,6 +57,7 @@ struct InOffsetsArgs {
     uint32_t *totals[2];
     uint32_t *block_sums[2];
     uint64_t *ofs[2];
+    uint64_t *few_report[2];   // optional (host-visible) word per stream: n_tiles << 32 | tiles none of whose blocks has more than three planes
 };
 hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, hipStream_t s);
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s);
