@@ -50,8 +50,7 @@ struct homcomp_workspace {
     uint64_t *d_tile_totals;   // [max_tiles]  output-offset scan: tile totals
     uint64_t *d_tile_prefixes; // [max_tiles]  output-offset scan: tile prefixes (adjacent to the totals)
     uint64_t *d_in_ofs[2];    // [max_tiles+1] tile payload offsets of the incoming streams
-    uint32_t *d_in_totals[2]; // [max_tiles]   scratch of the offsets pre-pass, per stream: tile totals
-    uint32_t *d_in_blocks[2]; // [max_tiles/256 + 1]  and sums over blocks of 256 tiles
+    uint64_t *d_in_blocks[2]; // [max_tiles/256 + 1]  words of the offsets pre-pass, per stream: totals of blocks of 256 tiles, tagged with the epoch
     uint64_t *d_total;        // stream length of the last stream-producing call
     uint32_t *d_error;        // sticky error flags, next to d_total
     float *d_partial;         // min/max partials
@@ -82,12 +81,15 @@ int check_ws(const homcomp_workspace *ws, size_t n)
     return HOMCOMP_OK;
 }
 
-// Fresh epoch for one launch; clears the scan words when the 22-bit tag wraps (the two arrays
-// are adjacent).
+// Fresh epoch for one launch; clears the scan words (the two arrays are adjacent) and the block
+// words of the offsets pre-pass when the 22-bit tag wraps.
 int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
 {
     if (ws->epoch >= kMaxEpoch) {
-        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)))
+        const uint64_t blocks = (uint64_t)ws->max_tiles / 256 + 1;
+        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)) ||
+            !hip_ok(hc::launch_fill_u64(ws->d_in_blocks[0], blocks, s)) ||
+            !hip_ok(hc::launch_fill_u64(ws->d_in_blocks[1], blocks, s)))
             return HOMCOMP_ERR_HIP;
         ws->epoch = 0;
     }
@@ -110,20 +112,31 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
 }
 
 // Offsets pre-pass of the incoming streams (header bytes -> payload offset of every tile): one
-// pass of launches for all of them.
+// launch for all of them, under the epoch of the call's tile kernel.
 int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s, bool report_few = false)
 {
     hc::InOffsetsArgs a;
     std::memset(&a, 0, sizeof a);
+    a.error = ws->d_error;
+    uint32_t epoch = p->epoch;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        // as for the tile kernel (see chained_launch): a replay finds the words of the replay before
+        (void)hipGetLastError();
+        epoch = kGraphEpoch;
+        const uint64_t blocks = (uint64_t)p->n_tiles / 256 + 1;
+        for (int c = 0; c < n_streams; ++c)
+            if (!hip_ok(hc::launch_fill_u64(ws->d_in_blocks[c], blocks, s))) return HOMCOMP_ERR_HIP;
+    }
     for (int c = 0; c < n_streams; ++c) {
         p->in_ofs[c] = ws->d_in_ofs[c];
         a.hdr[c] = p->in[c];
-        a.totals[c] = ws->d_in_totals[c];
-        a.block_sums[c] = ws->d_in_blocks[c];
+        a.block_words[c] = ws->d_in_blocks[c];
         a.ofs[c] = ws->d_in_ofs[c];
     }
     if (report_few) a.few_report[0] = ws->h_few;
-    return hip_ok(hc::launch_in_offsets(a, n_streams, p->n_tiles, p->hdr_bytes, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+    return hip_ok(hc::launch_in_offsets(a, n_streams, p->n_tiles, p->hdr_bytes, epoch, ws->spin_limit, s)) ? HOMCOMP_OK
+                                                                                                            : HOMCOMP_ERR_HIP;
 }
 
 // LDS stage per data wave (two deferred tiles by default), in three budgets that let 4, 3 and 2
@@ -316,10 +329,9 @@ constexpr uint32_t kStaticDataGroups = 224;   // data workgroups of four waves
 constexpr uint32_t kStaticSlots = 2;          // deferral depth
 constexpr size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr size_t kStaticOfsScan = 0;                                                                   // 2 x tiles words
-constexpr size_t kStaticOfsIn = kStaticOfsScan + align256(2 * (size_t)kStaticMaxTiles * 8);            // tiles + 1 offsets
-constexpr size_t kStaticOfsTotals = kStaticOfsIn + align256(((size_t)kStaticMaxTiles + 1) * 8);        // tiles totals
-constexpr size_t kStaticOfsBlocks = kStaticOfsTotals + align256((size_t)kStaticMaxTiles * 4);          // sums over 256 tiles
-constexpr size_t kStaticOfsSpill = kStaticOfsBlocks + align256(((size_t)kStaticMaxTiles / 256 + 1) * 4);
+constexpr size_t kStaticOfsIn = kStaticOfsScan + align256(2 * (size_t)kStaticMaxTiles * 8);            // tiles offsets
+constexpr size_t kStaticOfsBlocks = kStaticOfsIn + align256((size_t)kStaticMaxTiles * 8);              // words of blocks of 256 tiles
+constexpr size_t kStaticOfsSpill = kStaticOfsBlocks + align256(((size_t)kStaticMaxTiles / 256 + 1) * 8);
 constexpr size_t kStaticBytes =
     kStaticOfsSpill + (size_t)kStaticDataGroups * 4 * kStaticSlots * hc::kSpillSlotBytes;   // about 28.3 MiB
 
@@ -437,12 +449,10 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     size_t off = 0;
     auto take = [&off](size_t bytes) { size_t o = off; off = (off + bytes + 255) & ~(size_t)255; return o; };
     const size_t o_status = take(2 * t * sizeof(uint64_t));
-    const size_t o_in0 = take((t + 1) * sizeof(uint64_t));
-    const size_t o_in1 = take((t + 1) * sizeof(uint64_t));
-    const size_t o_tot0 = take(t * sizeof(uint32_t));
-    const size_t o_tot1 = take(t * sizeof(uint32_t));
-    const size_t o_blk0 = take((t / 256 + 1) * sizeof(uint32_t));
-    const size_t o_blk1 = take((t / 256 + 1) * sizeof(uint32_t));
+    const size_t o_in0 = take(t * sizeof(uint64_t));
+    const size_t o_in1 = take(t * sizeof(uint64_t));
+    const size_t o_blk0 = take((t / 256 + 1) * sizeof(uint64_t));
+    const size_t o_blk1 = take((t / 256 + 1) * sizeof(uint64_t));
     const size_t o_total = take(64);
     const size_t o_partial = take(kRangePartials * 2 * sizeof(float));
     const size_t bytes = off;
@@ -517,10 +527,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     ws->d_tile_prefixes = ws->d_tile_totals + t;
     ws->d_in_ofs[0] = (uint64_t *)(base + o_in0);
     ws->d_in_ofs[1] = (uint64_t *)(base + o_in1);
-    ws->d_in_totals[0] = (uint32_t *)(base + o_tot0);
-    ws->d_in_totals[1] = (uint32_t *)(base + o_tot1);
-    ws->d_in_blocks[0] = (uint32_t *)(base + o_blk0);
-    ws->d_in_blocks[1] = (uint32_t *)(base + o_blk1);
+    ws->d_in_blocks[0] = (uint64_t *)(base + o_blk0);
+    ws->d_in_blocks[1] = (uint64_t *)(base + o_blk1);
     ws->d_total = (uint64_t *)(base + o_total);
     ws->d_error = (uint32_t *)(base + o_total + 8);
     ws->d_partial = (float *)(base + o_partial);
@@ -743,17 +751,19 @@ int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size
     p.sliced = tile_bytes_of(p, cmp_in_size) <= kBitplaneTileBytes;
     const int cls = choose_stage_class(hc::kOpHomSumF32, tile_bytes_of(p, cmp_in_size), kStaticSlots);
     p.stage_bytes = kStage[cls][hc::kOpHomSumF32];
-    // totals and prefixes of the tiles this call uses (the arrays keep the last call's words)
-    if (!hip_ok(hc::launch_fill_u64(p.tile_totals, p.n_tiles, s)) ||
-        !hip_ok(hc::launch_fill_u64(p.tile_prefixes, p.n_tiles, s)))
-        return HOMCOMP_ERR_HIP;
+    // totals and prefixes of the tiles this call uses and the block words of its pre-pass (the
+    // arrays keep the last call's words)
     hc::InOffsetsArgs a;
     std::memset(&a, 0, sizeof a);
     a.hdr[0] = d_cmp_in;
-    a.totals[0] = (uint32_t *)(base + kStaticOfsTotals);
-    a.block_sums[0] = (uint32_t *)(base + kStaticOfsBlocks);
+    a.block_words[0] = (uint64_t *)(base + kStaticOfsBlocks);
     a.ofs[0] = (uint64_t *)(base + kStaticOfsIn);
-    if (!hip_ok(hc::launch_in_offsets(a, 1, p.n_tiles, p.hdr_bytes, s))) return HOMCOMP_ERR_HIP;
+    a.error = p.error;
+    if (!hip_ok(hc::launch_fill_u64(p.tile_totals, p.n_tiles, s)) ||
+        !hip_ok(hc::launch_fill_u64(p.tile_prefixes, p.n_tiles, s)) ||
+        !hip_ok(hc::launch_fill_u64(a.block_words[0], (uint64_t)p.n_tiles / 256 + 1, s)))
+        return HOMCOMP_ERR_HIP;
+    if (!hip_ok(hc::launch_in_offsets(a, 1, p.n_tiles, p.hdr_bytes, p.epoch, p.spin_limit, s))) return HOMCOMP_ERR_HIP;
     return chained_launch(device, nullptr, 0, hc::kOpHomSumF32, p, st->grid[cls], s);
 }
 

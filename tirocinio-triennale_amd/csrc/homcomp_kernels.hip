@@ -971,11 +971,16 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 // ---------------------------------------------------------------- incoming-stream offsets
 //
 // The payload offset of a tile of an incoming stream depends on the header bytes only
-// (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel in two fully parallel
-// steps over blocks of 256 tiles: k_in_totals sums the block sizes of every tile (16 header
-// bytes per lane) and leaves one sum per block; k_in_offsets adds up the sums of
-// the earlier blocks, scans the block's 256 totals and writes the tiles' absolute offsets
-// (`base` = header length).
+// (HomComp/src/GSZ.cu:790-874), so it is computed ahead of the tile kernel, in one launch over
+// blocks of 256 tiles: a workgroup sums the block sizes of each of its tiles (16 header bytes
+// per lane), publishes the block's total in the block's word, scans its 256 totals, adds up
+// the totals of the earlier blocks as they appear and writes the tiles' absolute offsets
+// (`base` = header length).  A workgroup only ever waits for workgroups with smaller indices,
+// which the hardware starts first, and every one of them publishes before it waits, so the
+// waits end whatever else runs on the device; they are bounded all the same (a wait that runs
+// into its bound raises the error flag, and the offsets it leaves are only ever used to read
+// within the stream's stated size).  The words carry the launch's epoch like the scan words of
+// the tile kernels, so they are never cleared between calls.
 
 constexpr uint32_t kOfsBlockTiles = 256;
 constexpr uint32_t kBlockSumBits = 23;
@@ -996,15 +1001,13 @@ __device__ __forceinline__ uint32_t wg_reduce_u32(uint32_t v, uint32_t *s_tmp)
     return t;
 }
 
-// A stream of at most one block of tiles (4 MiB of values) gets its offsets from k_in_totals
-// itself (`ofs` not null, one workgroup): the second launch would be a fifth of such a call.
 // One launch serves up to two streams (blockIdx.y), each with its own arrays.
-__global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base, int direct)
+__global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base,
+                                                    uint32_t epoch, uint32_t spin_limit)
 {
     const uint8_t *__restrict__ hdr = a.hdr[blockIdx.y];
-    uint32_t *__restrict__ totals = a.totals[blockIdx.y];
-    uint32_t *__restrict__ block_sums = a.block_sums[blockIdx.y];
-    uint64_t *__restrict__ ofs = direct ? a.ofs[blockIdx.y] : nullptr;
+    uint64_t *__restrict__ words = a.block_words[blockIdx.y];
+    uint64_t *__restrict__ ofs = a.ofs[blockIdx.y];
     __shared__ uint32_t s_tmp[4];
     __shared__ uint32_t s_tot[kOfsBlockTiles];
     uint32_t acc = 0, few_tiles = 0;
@@ -1054,10 +1057,7 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
         planes |= dpp_u32<kDppXor2>(planes);
         planes |= dpp_u32<kDppRowHalfMirror>(planes);
         if ((threadIdx.x & (kPieces - 1)) == 0) {
-            if (tile < n_tiles) {
-                totals[tile] = sum;
-                few_tiles += planes <= kFewPlanes ? 1u : 0u;
-            }
+            if (tile < n_tiles) few_tiles += planes <= kFewPlanes ? 1u : 0u;
             s_tot[tile % kOfsBlockTiles] = sum;   // 0 beyond the last tile
         }
     }
@@ -1065,10 +1065,10 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
     const uint32_t block_few = wg_reduce_u32(few_tiles, s_tmp);
     // a block's bytes stay below 2^23 (256 tiles of at most 128 * 132 bytes): its count of tiles
     // with few planes (at most 256) travels in the bits above
-    static_assert(kOfsBlockTiles * kTileBlocks * kMaxBlockBytes < (1u << kBlockSumBits), "packing of the block sums");
-    if (threadIdx.x == 0) block_sums[blockIdx.x] = block_total | (block_few << kBlockSumBits);
-    if (ofs == nullptr) return;
-    // one block of tiles: its offsets right away, as k_in_offsets below would compute them
+    static_assert(kOfsBlockTiles * kTileBlocks * kMaxBlockBytes < (1u << kBlockSumBits), "packing of the block totals");
+    if (threadIdx.x == 0) status_store(&words[blockIdx.x], status_word(epoch, 2u, block_total | (block_few << kBlockSumBits)));
+
+    // the block's own tiles
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t mine = s_tot[threadIdx.x];
     const uint32_t incl = wave_incl_scan_u32(mine, lane);
@@ -1076,53 +1076,41 @@ __global__ __launch_bounds__(256) void k_in_totals(const InOffsetsArgs a, uint32
     __syncthreads();
     uint32_t earlier = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-        if (q < wave) earlier += s_tmp[q];
-    if (threadIdx.x < n_tiles) ofs[threadIdx.x] = base + earlier + (incl - mine);
-    if (threadIdx.x == 0) {
-        ofs[n_tiles] = base + block_total;   // the end of the payload
-        if (a.few_report[blockIdx.y]) *a.few_report[blockIdx.y] = ((uint64_t)n_tiles << 32) | block_few;
-    }
-}
+    for (int w = 0; w < 4; ++w)
+        if (w < wave) earlier += s_tmp[w];
+    __syncthreads();
 
-__global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint32_t n_tiles, uint64_t base)
-{
-    const uint32_t *__restrict__ totals = a.totals[blockIdx.y];
-    const uint32_t *__restrict__ block_sums = a.block_sums[blockIdx.y];
-    uint64_t *__restrict__ ofs = a.ofs[blockIdx.y];
-    __shared__ uint32_t s_tmp[4];
-    __shared__ uint32_t s_wave[4];
-    // bytes of all earlier blocks (a block is at most 256 * 132 * 128 bytes, so 64-bit sums)
-    uint64_t before = 0;
-    uint32_t few_before = 0;
+    // the blocks before it, 256 at a time
     const bool last = (blockIdx.x + 1) * kOfsBlockTiles >= n_tiles;   // this block also reports the count of tiles with few planes
-    for (uint32_t q0 = 0; q0 < blockIdx.x + (last ? 1u : 0u); q0 += 256) {
-        const uint32_t q = q0 + threadIdx.x;
-        const uint32_t packed = q <= blockIdx.x ? block_sums[q] : 0u;
-        const uint32_t v = q < blockIdx.x ? packed & ((1u << kBlockSumBits) - 1u) : 0u;
+    uint64_t before = 0;
+    uint32_t few_before = block_few;
+    bool ok = true;
+    for (uint32_t q0 = 0; q0 < blockIdx.x; q0 += 256) {
+        const uint32_t b = q0 + threadIdx.x;
+        uint32_t packed = 0;
+        if (b < blockIdx.x) {
+            uint64_t w = status_load(&words[b]);
+            uint32_t spins = 0;
+            while (ok && status_state(w, epoch) != 2u) {
+                if (++spins > spin_limit) {
+                    ok = false;   // and no further waiting in this launch
+                } else {
+                    __builtin_amdgcn_s_sleep(2);
+                    w = status_load(&words[b]);
+                }
+            }
+            packed = ok ? (uint32_t)w : 0u;
+        }
+        const uint32_t v = packed & ((1u << kBlockSumBits) - 1u);
         // split so that the 32-bit reduction cannot overflow (256 values below 2^23 each)
         before += (uint64_t)wg_reduce_u32(v & 0xffffu, s_tmp) + ((uint64_t)wg_reduce_u32(v >> 16, s_tmp) << 16);
-        if (last) few_before += wg_reduce_u32(packed >> kBlockSumBits, s_tmp);   // its own block included
+        if (last) few_before += wg_reduce_u32(packed >> kBlockSumBits, s_tmp);
     }
+    if (!ok) atomicOr(a.error, 1u);
     const uint32_t tile = blockIdx.x * kOfsBlockTiles + threadIdx.x;
-    const uint32_t mine = tile < n_tiles ? totals[tile] : 0u;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t incl = wave_incl_scan_u32(mine, lane);
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t earlier = 0, block_total = 0;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t t = s_wave[q];
-        if (q < wave) earlier += t;
-        block_total += t;
-    }
     if (tile < n_tiles) ofs[tile] = base + before + earlier + (incl - mine);
-    // the entry after the last tile is the end of the payload
-    if (threadIdx.x == 0 && last) {
-        ofs[n_tiles] = base + before + block_total;
-        if (a.few_report[blockIdx.y]) *a.few_report[blockIdx.y] = ((uint64_t)n_tiles << 32) | few_before;
-    }
+    if (threadIdx.x == 0 && last && a.few_report[blockIdx.y])
+        *a.few_report[blockIdx.y] = ((uint64_t)n_tiles << 32) | few_before;
 }
 
 // HomComp/src/homcomp.cu:1553-1602: Lorenzo deltas of the quantised values as int32.
@@ -1313,15 +1301,11 @@ hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t
     }
 }
 
-hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, hipStream_t s)
+hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, uint32_t epoch,
+                             uint32_t spin_limit, hipStream_t s)
 {
     const uint32_t blocks = (n_tiles + kOfsBlockTiles - 1) / kOfsBlockTiles;
-    if (blocks == 1) {
-        hipLaunchKernelGGL(k_in_totals, dim3(1, n_streams), dim3(256), 0, s, a, n_tiles, base, 1);
-        return hipGetLastError();
-    }
-    hipLaunchKernelGGL(k_in_totals, dim3(blocks, n_streams), dim3(256), 0, s, a, n_tiles, (uint64_t)0, 0);
-    hipLaunchKernelGGL(k_in_offsets, dim3(blocks, n_streams), dim3(256), 0, s, a, n_tiles, base);
+    hipLaunchKernelGGL(k_in_offsets, dim3(blocks, n_streams), dim3(256), 0, s, a, n_tiles, base, epoch, spin_limit);
     return hipGetLastError();
 }
 

@@ -19,7 +19,7 @@ constexpr uint32_t kHostChunkElems = 32768;
 struct TileParams {
     const uint8_t *in[2];       // incoming streams (header + payload)
     uint64_t in_size[2];        // their stated sizes (out-of-bound rule)
-    const uint64_t *in_ofs[2];  // per stream: absolute payload offset of every tile, n_tiles + 1 entries
+    const uint64_t *in_ofs[2];  // per stream: absolute payload offset of every tile
     const void *local;          // float32 values or int32 deltas, n elements, 16-byte aligned
     uint8_t *out_cmp;           // outgoing stream
     float *out_f32;             // decompressed values
@@ -50,16 +50,17 @@ constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
 hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu);
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
 // Tile payload offsets of one or two incoming streams (of the same length) from their header
-// bytes, in one pass of launches: per stream the header bytes, two scratch arrays (n_tiles totals,
-// n_tiles / 256 + 1 sums) and the n_tiles + 1 offsets to be written.
+// bytes, in one launch.
 struct InOffsetsArgs {
-    const uint8_t *hdr[2];
-    uint32_t *totals[2];
-    uint32_t *block_sums[2];
-    uint64_t *ofs[2];
-    uint64_t *few_report[2];   // optional (host-visible) word per stream: n_tiles << 32 | tiles none of whose blocks has more than three planes
+    const uint8_t *hdr[2];      // the streams' header bytes
+    uint64_t *block_words[2];   // per stream and block of 256 tiles: a word tagged with the launch's epoch, n_tiles / 256 + 1 of them
+    uint64_t *ofs[2];           // result: absolute payload offset of every tile
+    uint64_t *few_report[2];    // optional (host-visible) word per stream: n_tiles << 32 | tiles none of whose blocks has more than three planes
+    uint32_t *error;            // sticky error flags (bit 0: a bounded wait gave up)
 };
-hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, hipStream_t s);
+// `epoch`: as TileParams::epoch, any value the block words have not seen since they were last cleared.
+hipError_t launch_in_offsets(const InOffsetsArgs &a, int n_streams, uint32_t n_tiles, uint64_t base, uint32_t epoch,
+                             uint32_t spin_limit, hipStream_t s);
 hipError_t launch_quant_predict(const float *x, int32_t *out, uint64_t n, float recip, hipStream_t s);
 hipError_t launch_range(const float *x, uint64_t n, float *partial, uint32_t max_partials,
                         float *out, hipStream_t s);
