@@ -32,7 +32,8 @@ def measured_traffic(kind: str, log2n: int, rel: float):
     workload (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, two runs), with the scaling that summary
     states; None when no summary of the workload is there."""
     size = f"{4 * (1 << log2n) // 2**30}GiB" if log2n >= 28 else f"{4 * (1 << log2n) // 2**20}MiB"
-    path = os.path.join(PROFILES, f"pmc_hbm_traffic_{kind}_{size}_rel{rel:g}.txt")
+    bound = f"{rel:.0e}".replace("e-0", "e-")   # 1e-4
+    path = os.path.join(PROFILES, f"pmc_hbm_traffic_{kind}_{size}_rel{bound}.txt")
     try:
         with open(path) as f:
             for line in f:
