@@ -178,9 +178,40 @@ struct DeviceState {
     size_t spill_bytes = 0;
     int spill_users = 0;
     std::vector<void *> retired;
+    // persistent grid of each operation's kernel per LDS budget, at 100 percent; worked out once
+    bool grids_ready = false;
+    uint32_t full_grid[hc::kOpCount][kStageClasses];
 };
 constexpr int kMaxDevices = 64;
 DeviceState g_dev[kMaxDevices];
+
+// Resident grid of every operation and LDS budget on `device` (the current device), computed once
+// per process: the occupancy queries set a limit that belongs to the kernel function, which must
+// not change while other host threads launch.
+int device_grids(int device, const uint32_t (**grids)[kStageClasses])
+{
+    DeviceState &d = g_dev[device];
+    std::lock_guard<std::mutex> lock(d.mu);
+    *grids = d.full_grid;
+    if (d.grids_ready) return HOMCOMP_OK;
+    hipDeviceProp_t prop;
+    if (!hip_ok(hipGetDeviceProperties(&prop, device))) return HOMCOMP_ERR_HIP;
+    // one compute unit's worth of workgroups is left free: the persistent grid must be fully
+    // resident, and an estimate that is off by a single workgroup would stall the launch
+    const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
+    for (int op = 0; op < hc::kOpCount; ++op) {
+        for (int cls = 0; cls < kStageClasses; ++cls) {
+            int per_cu = 0;
+            const uint32_t stage = op == hc::kOpDecompress ? 0u : kStage[cls][op];
+            const uint32_t largest = op == hc::kOpDecompress ? 0u : kStage[kStageClasses - 1][op];
+            if (!hip_ok(hc::op_kernel_residency(op, stage, largest, &per_cu))) return HOMCOMP_ERR_HIP;
+            if (per_cu < 1) per_cu = 1;
+            d.full_grid[op][cls] = (uint32_t)per_cu * (uint32_t)cus;
+        }
+    }
+    d.grids_ready = true;
+    return HOMCOMP_OK;
+}
 
 int spill_acquire(homcomp_workspace *ws, size_t bytes)
 {
@@ -362,14 +393,10 @@ int static_setup(int device, StaticState **out)
     if (st.ready) return HOMCOMP_OK;
     void *ptr = nullptr;
     if (!hip_ok(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) || !ptr) return HOMCOMP_ERR_HIP;
-    hipDeviceProp_t prop;
-    if (!hip_ok(hipGetDeviceProperties(&prop, device))) return HOMCOMP_ERR_HIP;
+    const uint32_t (*grids)[kStageClasses] = nullptr;
+    if (device_grids(device, &grids) != HOMCOMP_OK) return HOMCOMP_ERR_HIP;
     for (int cls = 0; cls < kStageClasses; ++cls) {
-        int per_cu = 0;
-        if (!hip_ok(hc::op_kernel_residency(hc::kOpHomSumF32, kStage[cls][hc::kOpHomSumF32], &per_cu))) return HOMCOMP_ERR_HIP;
-        if (per_cu < 1) per_cu = 1;
-        const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
-        uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
+        uint32_t g = grids[hc::kOpHomSumF32][cls];
         if (g > kStaticDataGroups + 1) g = kStaticDataGroups + 1;   // the spill area holds this many groups
         if (g < 2) g = 2;
         st.grid[cls] = g;
@@ -456,19 +483,12 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     const size_t o_total = take(64);
     const size_t o_partial = take(kRangePartials * 2 * sizeof(float));
     const size_t bytes = off;
-    hipDeviceProp_t prop;
-    bool ok = hip_ok(hipGetDeviceProperties(&prop, ws->device));
+    const uint32_t (*grids)[kStageClasses] = nullptr;
+    bool ok = device_grids(ws->device, &grids) == HOMCOMP_OK;
     uint32_t widest = 0;
     for (int op = 0; ok && op < hc::kOpCount; ++op) {
-        for (int cls = 0; ok && cls < kStageClasses; ++cls) {
-            int per_cu = 0;
-            const uint32_t stage = op == hc::kOpDecompress ? 0u : kStage[cls][op];
-            ok = hip_ok(hc::op_kernel_residency(op, stage, &per_cu));
-            if (ok && per_cu < 1) per_cu = 1;
-            // one compute unit's worth of workgroups is left free: the persistent grid must be fully
-            // resident, and an estimate that is off by a single workgroup would stall the launch
-            const int cus = prop.multiProcessorCount > 1 ? prop.multiProcessorCount - 1 : 1;
-            const uint32_t g = (uint32_t)per_cu * (uint32_t)cus;
+        for (int cls = 0; cls < kStageClasses; ++cls) {
+            const uint32_t g = grids[op][cls];
             ws->full_grid[op][cls] = g;
             if (op != hc::kOpDecompress && g > widest) widest = g;
         }

@@ -1238,11 +1238,15 @@ static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_
 }
 
 template <int NIN, int LOCAL, int OUT, bool BITPLANE>
-static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
+static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes, uint32_t max_stage_bytes)
 {
     const size_t dyn = OUT == kOutStream ? (size_t)(kWG / 64) * stage_bytes : 0;
+    const size_t max_dyn = OUT == kOutStream ? (size_t)(kWG / 64) * max_stage_bytes : 0;
     const void *fn = reinterpret_cast<const void *>(&k_wave<NIN, LOCAL, OUT, BITPLANE>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+    // The limit on the kernel's dynamic LDS belongs to the function, not to a launch: it is only
+    // ever set to the largest budget, because another host thread may be launching the kernel
+    // with any budget at this moment (a limit lowered for the query made such a launch fail).
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_dyn);
     if (e != hipSuccess) return e;
     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, k_wave<NIN, LOCAL, OUT, BITPLANE>, kWG, dyn);
     // The stream-producing kernels need every workgroup of the grid resident at the same time
@@ -1264,23 +1268,24 @@ static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
 
 // both kinds of a kernel: the smaller of the two answers
 template <int NIN, int LOCAL, int OUT>
-static hipError_t both_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes)
+static hipError_t both_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes, uint32_t max_stage_bytes)
 {
     int with = 0, without = 0;
-    hipError_t e = wave_resident_blocks<NIN, LOCAL, OUT, true>(&with, stage_bytes);
-    if (e == hipSuccess) e = wave_resident_blocks<NIN, LOCAL, OUT, false>(&without, stage_bytes);
+    hipError_t e = wave_resident_blocks<NIN, LOCAL, OUT, true>(&with, stage_bytes, max_stage_bytes);
+    if (e == hipSuccess) e = wave_resident_blocks<NIN, LOCAL, OUT, false>(&without, stage_bytes, max_stage_bytes);
     *blocks_per_cu = with < without ? with : without;
     return e;
 }
 
-hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu)
+hipError_t op_kernel_residency(int op, uint32_t stage_bytes, uint32_t max_stage_bytes, int *blocks_per_cu)
 {
+    if (stage_bytes > max_stage_bytes) return hipErrorInvalidValue;
     switch (op) {
-    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream, false>(blocks_per_cu, stage_bytes);
-    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32, false>(blocks_per_cu, stage_bytes);
-    case kOpHomSumF32: return both_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes);
-    case kOpHomSumI32: return both_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes);
-    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream, true>(blocks_per_cu, stage_bytes);
+    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream, false>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32, false>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomSumF32: return both_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomSumI32: return both_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream, true>(blocks_per_cu, stage_bytes, max_stage_bytes);
     default: return hipErrorInvalidValue;
     }
 }

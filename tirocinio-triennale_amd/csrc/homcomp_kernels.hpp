@@ -46,8 +46,10 @@ struct TileParams {
 
 // Bytes per slot of the spill area (TileParams::spill): a whole worst-case tile.
 constexpr uint32_t kSpillSlotBytes = kHostTileBlocks * 128u + 128u;
-// Resident workgroups per compute unit of the kernel behind an operation (sizes the persistent grid).
-hipError_t op_kernel_residency(int op, uint32_t stage_bytes, int *blocks_per_cu);
+// Resident workgroups per compute unit of the kernel behind an operation with `stage_bytes` of
+// LDS stage per data wave (sizes the persistent grid).  `max_stage_bytes`: the largest stage any
+// launch of the operation uses; the kernel's limit on dynamic LDS is set to that.
+hipError_t op_kernel_residency(int op, uint32_t stage_bytes, uint32_t max_stage_bytes, int *blocks_per_cu);
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s);
 // Tile payload offsets of one or two incoming streams (of the same length) from their header
 // bytes, in one launch.
