@@ -440,7 +440,8 @@ def main() -> int:
                 "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ops[dom]["frac_hbm"],
                 "traffic": traffic["bytes"] if traffic and traffic["kernel"] == dom else None,
                 "traffic_calibration": traffic["calibration"] if traffic else None,
-                "traffic_source": traffic["source"] if traffic else None}
+                "traffic_source": traffic["source"] if traffic else None,
+                "timed": "whole hom_sum_f32 call (offsets pre-pass k_in_offsets + tile kernel k_wave), HIP events on the call's stream"}
 
     out = {
         "metric": "compress + hom-add throughput (GB/s of uncompressed input)",

@@ -539,6 +539,52 @@ def test_two_streams_do_not_overlap_their_scans(pkg, cuda, orc, gen):
         assert_stream_equal(out2[1][:L2].cpu().numpy(), want_sum, "hom_sum_f32 on stream 2")
 
 
+def test_workspaces_created_while_other_threads_launch(pkg, cuda, orc, gen):
+    """One workspace per host thread, created, used on a stream of its own (compress with the
+    large LDS budget of a first call, then stream (+) floats) and destroyed while the other
+    threads do the same: the occupancy queries of a creation set
+    a limit that belongs to the kernel function, and a launch from another thread must never see it
+    lowered.  Every thread must get the oracle's bytes and no error."""
+    import threading
+    torch = cuda
+    orc.set_threads(16)
+    n = (1 << 18) + 4096 + 5
+    eb = np.float32(8e-4)
+    a, b = gen.smooth_np(n, 81), gen.smooth_np(n, 82)
+    want_a = orc.compress(a, eb)
+    want_s = orc.hom_sum_f32(want_a, b, eb)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    cap = pkg.max_stream_bytes(n)
+    torch.cuda.synchronize()
+    errors = []
+
+    def rank(r):
+        try:
+            stream = torch.cuda.Stream()
+            out = torch.empty(cap, dtype=torch.uint8, device="cuda")
+            out2 = torch.empty(cap, dtype=torch.uint8, device="cuda")
+            for it in range(6):
+                with pkg.Workspace(n) as ws:
+                    ws.compress(da, float(eb), out, stream=stream)
+                    la = ws.last_size(stream=stream)
+                    ws.hom_sum_f32(out, la, db, float(eb), out2, stream=stream)
+                    ls = ws.last_size(stream=stream)
+                    if la != want_a.size or not np.array_equal(out[:la].cpu().numpy(), want_a):
+                        errors.append(f"thread {r}, round {it}: compress differs")
+                    if ls != want_s.size or not np.array_equal(out2[:ls].cpu().numpy(), want_s):
+                        errors.append(f"thread {r}, round {it}: hom_sum_f32 differs")
+        except Exception as e:   # a failed launch arrives here as HomCompError
+            errors.append(f"thread {r}: {e!r}")
+
+    threads = [threading.Thread(target=rank, args=(r,)) for r in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors[:4]
+
+
 def test_graph_replay(pkg, cuda, orc, gen):
     """compress, hom_sum_f32 and decompress captured into one HIP graph (no call allocates or
     blocks when the lengths go to device words) and replayed with new operand contents, with
