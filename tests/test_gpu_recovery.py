@@ -50,6 +50,55 @@ def test_scan_timeout_is_reported_once_and_the_workspace_recovers(pkg, cuda, orc
         g.close()
 
 
+def test_timeouts_with_an_incoming_stream(pkg, cuda, orc, gen):
+    """The same with an incoming stream, whose offsets pre-pass has bounded waits of its own (a
+    block of tiles waits for the totals of the blocks before it): with the bound at zero the
+    pre-pass may leave offsets that are too small and the tile kernel gives up as above; nothing
+    is read beyond the stated size plus its slack or written outside the output buffers, the
+    error is reported once, and the workspace recovers."""
+    torch = cuda
+    orc.set_threads(16)
+    n = 1 << 24                      # 4096 tiles, 16 blocks of tiles in the pre-pass
+    eb = np.float32(8e-4)
+    x, y = gen.smooth_np(n, 151), gen.smooth_np(n, 152)
+    sa = orc.compress(x, eb)
+    want = orc.hom_sum_f32(sa, y, eb)
+    want_dec = orc.decompress(want, n, eb)
+    dy = torch.from_numpy(y).cuda()
+    cap = pkg.max_stream_bytes(n)
+    guard = 4096
+    src = torch.zeros(cap + 256, dtype=torch.uint8, device="cuda")
+    src[:sa.size] = torch.from_numpy(sa).cuda()
+    buf = torch.full((cap + 2 * guard,), 0xC3, dtype=torch.uint8, device="cuda")
+    out = buf[guard:guard + cap]
+    fbuf = torch.full((n + 2 * guard,), 7.0, dtype=torch.float32, device="cuda")
+    dec = fbuf[guard:guard + n]
+    with pkg.Workspace(n) as ws:
+        ws.set_option(pkg.OPT_SPIN_LIMIT, 0)
+        ws.hom_sum_f32(src, sa.size, dy, float(eb), out)
+        with pytest.raises(pkg.HomCompError) as info:
+            ws.last_size()
+        assert info.value.status == pkg.ERR_SCAN_TIMEOUT
+        # the decoder has no scan of its own, only the pre-pass can give up: either outcome is fine
+        ws.decompress(src, sa.size, n, float(eb), dec)
+        try:
+            ws.last_size()
+        except pkg.HomCompError as e:
+            assert e.status == pkg.ERR_SCAN_TIMEOUT
+        torch.cuda.synchronize()
+        assert bool((buf[:guard] == 0xC3).all()) and bool((buf[guard + cap:] == 0xC3).all())
+        assert bool((fbuf[:guard] == 7.0).all()) and bool((fbuf[guard + n:] == 7.0).all())
+        ws.last_size()                # clean: the failures above have been reported
+        ws.set_option(pkg.OPT_SPIN_LIMIT, 1 << 16)
+        ws.hom_sum_f32(src, sa.size, dy, float(eb), out)
+        L = ws.last_size()
+        got = out[:L].cpu().numpy()
+        assert L == want.size and np.array_equal(got, want), first_diff(got, want)
+        ws.decompress(out, L, n, float(eb), dec)
+        torch.cuda.synchronize()
+        assert np.array_equal(dec.cpu().numpy().view(np.uint32), want_dec.view(np.uint32))
+
+
 def test_set_option_rejects_bad_values(pkg, cuda):
     with pkg.Workspace(1 << 15) as ws:
         L = pkg.lib()
