@@ -1061,12 +1061,15 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
             s_tot[tile % kOfsBlockTiles] = sum;   // 0 beyond the last tile
         }
     }
-    const uint32_t block_total = wg_reduce_u32(acc, s_tmp);   // with a barrier: s_tot is complete
-    const uint32_t block_few = wg_reduce_u32(few_tiles, s_tmp);
     // a block's bytes stay below 2^23 (256 tiles of at most 128 * 132 bytes): its count of tiles
-    // with few planes (at most 256) travels in the bits above
+    // with few planes (at most 256) travels in the bits above, through the reduction as well
     static_assert(kOfsBlockTiles * kTileBlocks * kMaxBlockBytes < (1u << kBlockSumBits), "packing of the block totals");
-    if (threadIdx.x == 0) status_store(&words[blockIdx.x], status_word(epoch, 2u, block_total | (block_few << kBlockSumBits)));
+    const uint32_t block_packed = wg_reduce_u32(acc | (few_tiles << kBlockSumBits), s_tmp);   // with a barrier: s_tot is complete
+    const uint32_t block_few = block_packed >> kBlockSumBits;
+    if (threadIdx.x == 0) status_store(&words[blockIdx.x], status_word(epoch, 2u, block_packed));
+    // a first look at the words of the blocks before this one, on its way during the scan below
+    uint64_t first_look = 0;
+    if (threadIdx.x < blockIdx.x) first_look = status_load(&words[threadIdx.x]);
 
     // the block's own tiles
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1089,7 +1092,7 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
         const uint32_t b = q0 + threadIdx.x;
         uint32_t packed = 0;
         if (b < blockIdx.x) {
-            uint64_t w = status_load(&words[b]);
+            uint64_t w = q0 == 0 ? first_look : status_load(&words[b]);
             uint32_t spins = 0;
             while (ok && status_state(w, epoch) != 2u) {
                 if (++spins > spin_limit) {
@@ -1101,9 +1104,9 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
             }
             packed = ok ? (uint32_t)w : 0u;
         }
-        const uint32_t v = packed & ((1u << kBlockSumBits) - 1u);
-        // split so that the 32-bit reduction cannot overflow (256 values below 2^23 each)
-        before += (uint64_t)wg_reduce_u32(v & 0xffffu, s_tmp) + ((uint64_t)wg_reduce_u32(v >> 16, s_tmp) << 16);
+        // 256 values below 2^23 each: the sum fits 32 bits (the counts are summed apart: the byte
+        // totals of 256 blocks would carry into them)
+        before += wg_reduce_u32(packed & ((1u << kBlockSumBits) - 1u), s_tmp);
         if (last) few_before += wg_reduce_u32(packed >> kBlockSumBits, s_tmp);
     }
     if (!ok) atomicOr(a.error, 1u);
