@@ -338,6 +338,18 @@ __device__ __forceinline__ void unpack_low4(const uint8_t *stage, uint32_t base,
     }
 }
 
+// Sizes (size_from_header) and digests (header_digest, below) of two header bytes at once, a
+// byte each in the results: the same byte-parallel arithmetic as add_sizes_from_4_headers.
+__device__ __forceinline__ void sizes_and_digests_of_2_headers(uint32_t w, uint32_t &sizes, uint32_t &digests)
+{
+    const uint32_t F = w & 0x1f1fu;
+    const uint32_t sel = (w >> 7) & 0x0101u;
+    const uint32_t has_planes = ((F + 0x7f7fu) >> 7) & 0x0101u;   // F != 0
+    const uint32_t ob = (((w >> 5) & 0x0303u) + 0x0101u) & (sel * 0xffu);
+    sizes = (F << 2) + ((has_planes | sel) << 2) + ob;
+    digests = F | (ob << 5);
+}
+
 // What the decoder needs of a header byte, in one byte: bits 0-4 the plane count F, bits 5-7 the
 // number of outlier bytes (0 in plain mode, 1-4 in outlier mode).  0 for a block without payload.
 __device__ __forceinline__ uint32_t header_digest(uint32_t h)

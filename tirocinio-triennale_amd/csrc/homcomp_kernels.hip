@@ -420,8 +420,9 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             if (tile_of(r) < n_tiles) {
 #pragma unroll
                 for (int c = 0; c < NIN; ++c) {
-                    const uint32_t h0 = hdr_next[c] & 0xffu, h1 = hdr_next[c] >> 8;
-                    const uint32_t z0 = size_from_header(h0), z1 = size_from_header(h1);
+                    uint32_t sizes, digests;
+                    sizes_and_digests_of_2_headers(hdr_next[c], sizes, digests);
+                    const uint32_t z0 = sizes & 0xffu, z1 = sizes >> 8;
                     const uint32_t incl = wave_incl_scan_u32(z0 + z1, lane);
                     const uint32_t o0 = incl - z0 - z1, o1 = o0 + z0;
                     *reinterpret_cast<uint32_t *>(&s_ofs_in[wave][c][b][2 * lane]) = o0 | (o1 << 16);
@@ -432,8 +433,8 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     // what the sub-steps need of the header bytes; a block without payload, or one
                     // that starts at or beyond the stated size (out-of-bound rule of
                     // HomComp/src/GSZ.cu:908-911 on the absolute payload offset), is not read
-                    const uint32_t d0 = z0 != 0u && o0 < room ? header_digest(h0) : 0u;
-                    const uint32_t d1 = z1 != 0u && o1 < room ? header_digest(h1) : 0u;
+                    const uint32_t d0 = z0 != 0u && o0 < room ? digests & 0xffu : 0u;
+                    const uint32_t d1 = z1 != 0u && o1 < room ? digests >> 8 : 0u;
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
                     if constexpr (kAnySliced) {
                         // stream (+) stream takes tiles of up to kSlicedMaxF planes, stream (+) local operand of up to kFewPlanes
