@@ -458,7 +458,8 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         return HOMCOMP_ERR_NO_DEVICE;
     }
     const size_t tiles = padded_len(max_nbEle) / hc::kHostTileElems;
-    if (tiles >= (1ull << 31)) return HOMCOMP_ERR_TOO_LARGE;
+    // the kernels count tiles in 32 bits, with room for a few rounds of the grid beyond the last tile
+    if (tiles >= (1ull << 31) - (1ull << 16)) return HOMCOMP_ERR_TOO_LARGE;
     homcomp_workspace *ws = new (std::nothrow) homcomp_workspace();
     if (!ws) return HOMCOMP_ERR_INVALID_ARG;
     std::memset(ws, 0, sizeof *ws);

@@ -331,6 +331,12 @@ __device__ __forceinline__ void copy_out_spill(const uint8_t *slot, uint8_t *g, 
     if ((uint32_t)lane < tail) g[head + 16u * nch + lane] = byte_at(head + 16u * nch + (uint32_t)lane);
 }
 
+// Tile and round indices inside a launch.  32-bit arithmetic keeps the comparisons against the
+// tile count scalar, which the kernels with incoming streams (short of scalar registers) gain 1-3 %
+// from; compress, which has registers to spare, came out 1.7 % slower with it and keeps 64 bits.
+template <int NIN> struct TileIndex { typedef int32_t type; };
+template <> struct TileIndex<0> { typedef int64_t type; };
+
 // Registers of one incoming stream that travel ahead of the computation.
 struct InRegs {
     u32x4 chunk;   // the lane's 16-byte chunk of a sub-step's payload range
@@ -375,21 +381,24 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     const int lane = threadIdx.x & 63;
     const int k = lane & 3;
     const int quad = lane >> 2;
-    const int64_t n_tiles = p.n_tiles;
+    // tile indices are 32-bit: a launch has fewer than 2^31 - 2^15 tiles (the host checks), so
+    // tile + D * waves stays below 2^31 and the comparisons are scalar instructions
+    typedef typename TileIndex<NIN>::type tidx;
+    const tidx n_tiles = (tidx)p.n_tiles;
     const ScanCtx scan{p.tile_totals, p.tile_prefixes, p.n_tiles, p.epoch, p.spin_limit, p.error};
     // on the encoder the last workgroup of the grid is the scan server
-    const int64_t G = kEnc ? (int64_t)gridDim.x - 1 : (int64_t)gridDim.x;
-    const int64_t GW = G * kW;   // data waves
+    const tidx G = kEnc ? (tidx)gridDim.x - 1 : (tidx)gridDim.x;
+    const tidx GW = G * kW;   // data waves
     if constexpr (kEnc) {
-        if ((int64_t)blockIdx.x == G) {
-            scan_server(p, scan, (uint32_t)(GW < 0x7fffffff ? GW : 0x7fffffff));
+        if ((tidx)blockIdx.x == G) {
+            scan_server(p, scan, (uint32_t)GW);
             return;
         }
     }
-    const int64_t wid = (int64_t)blockIdx.x * kW + wave;
+    const tidx wid = (tidx)blockIdx.x * kW + wave;
     if (wid >= n_tiles) return;   // no barrier in this kernel: a wave without work just leaves
 
-    auto tile_of = [&](int64_t r) { return wid + r * GW; };
+    auto tile_of = [&](tidx r) { return wid + r * GW; };
 
     // ---- incoming streams: per-tile context
     uint32_t hdr_next[kIn];     // header bytes of blocks 2*lane, 2*lane+1 of the next tile
@@ -400,9 +409,9 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     uint32_t room_ctx0[kIn], room_ctx1[kIn];
     uint32_t end_ctx0[kIn], end_ctx1[kIn];   // payload bytes of those tiles
     uint32_t few_ctx = 0;   // bit-plane paths: bit b set = the blocks of the tile in context b (any stream) have few enough planes for them
-    auto fetch_headers = [&](int64_t r) __attribute__((always_inline)) {
+    auto fetch_headers = [&](tidx r) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
-            int64_t t = tile_of(r);
+            tidx t = tile_of(r);
             if (t >= n_tiles) t = 0;   // loads are issued unconditionally; the values are not used then
 #pragma unroll
             for (int c = 0; c < NIN; ++c) {
@@ -415,7 +424,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
         }
     };
     // header bytes -> block offsets of tile r in context buffer r & 1 (HomComp/src/GSZ.cu:790-874)
-    auto prepare = [&](int64_t r, int b) __attribute__((always_inline)) {
+    auto prepare = [&](tidx r, int b) __attribute__((always_inline)) {
         if constexpr (NIN > 0) {
             if (tile_of(r) < n_tiles) {
 #pragma unroll
@@ -483,12 +492,12 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     // staged the chunk, and the request for the sub-step after the next one is issued right there:
     // as early as possible, and ahead of the sub-step's own stores (a wave's memory operations
     // complete in order, so a load is only as fast as the stores issued before it).
-    auto request_local = [&](int64_t r, int s, SubRegs<LOCAL> &loc) __attribute__((always_inline)) {
-        const int64_t t = tile_of(r);
+    auto request_local = [&](tidx r, int s, SubRegs<LOCAL> &loc) __attribute__((always_inline)) {
+        const tidx t = tile_of(r);
         load_sub<LOCAL>(loc, p.local, p.n, (uint64_t)t * kTileElems, t < n_tiles, s, lane);
     };
     // (`wanted` false: nothing is read, the registers are only given a value)
-    auto request_in = [&](int c, int64_t r, int b, int s, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
+    auto request_in = [&](int c, tidx r, int b, int s, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
         if constexpr (kSliced) {
             if (!wanted) {   // wave-uniform; cheaper here than a request that fetches nothing
                 in[c].chunk = u32x4{0u, 0u, 0u, 0u};
@@ -503,7 +512,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             buffer_of(reinterpret_cast<const void *>(ga), wanted && tile_of(r) < n_tiles ? (nbytes + 15u) & ~15u : 0u);
         in[c].chunk = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, 0, kBufCached);
     };
-    auto request = [&](int64_t r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
+    auto request = [&](tidx r, int b, int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
         request_local(r, s, loc);
         if constexpr (NIN > 0) {
 #pragma unroll
@@ -588,10 +597,10 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     uint32_t spl[4] = {0, 0, 0, 0};     // how many of their first bytes lie in the spill slot (the rest in the LDS slot)
     uint64_t probe = 0;                // prefix word of the oldest one, requested a round ago
 
-    for (int64_t r = 0;; ++r) {
-        const int64_t t0 = tile_of(r);
-        const int64_t tp = t0 - (int64_t)(D - 1) * GW;   // its prefix is requested at the end of this round
-        const int64_t td = t0 - (int64_t)D * GW;         // copied out at the start of this round
+    for (tidx r = 0;; ++r) {
+        const tidx t0 = tile_of(r);
+        const tidx tp = t0 - (tidx)(D - 1) * GW;   // its prefix is requested at the end of this round
+        const tidx td = t0 - (tidx)D * GW;         // copied out at the start of this round
         const bool v0 = t0 < n_tiles;
         const bool vp = kEnc && r >= D - 1 && tp < n_tiles;
         const bool vd = kEnc && r >= D && td < n_tiles;
@@ -714,7 +723,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                 }
             };
             // `ahead` false: the registers are not sent out again (a sub-step run out of turn)
-            auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], int64_t r2, int b2, int s2, bool ahead = true)
+            auto sub = [&](int s, SubRegs<LOCAL> &loc, InRegs (&in)[kIn], tidx r2, int b2, int s2, bool ahead = true)
                            __attribute__((always_inline)) {
                 // the blocks' digests and offsets first: nothing in the sub-step writes them, and
                 // read here they are on their way while the wave waits for its operands
