@@ -26,7 +26,8 @@
  *   - An INPUT stream buffer must be readable up to cmp_size + 160 bytes (or up to
  *     homcomp_max_stream_bytes(nbEle), whichever is smaller): a block whose payload starts below
  *     the stated size is fetched in full (the out-of-bound rule of src/GSZ.cu:908-911 looks at the
- *     block's start only), in whole 16-byte pieces.  Buffers of homcomp_max_stream_bytes always do.
+ *     block's start only), in whole 16-byte pieces.  Buffers of homcomp_max_stream_bytes(nbEle) +
+ *     HOMCOMP_STREAM_SLACK bytes always do.
  *   - Stream-producing kernels keep their whole grid resident and wait for each other's scan
  *     words, so the library orders such launches of one process on a device, also across
  *     streams.  Launches recorded into a HIP graph are outside that order: a replay must not
@@ -66,6 +67,10 @@ size_t homcomp_header_bytes(size_t nbEle);
 /* Worst-case stream length: header + 128 payload bytes per block.  (The reference allocates
  * only 4*nbEle, src/homcomp_eval.cu:176, which incompressible input can overrun.) */
 size_t homcomp_max_stream_bytes(size_t nbEle);
+/* Bytes an INPUT stream buffer must be readable beyond the stream's stated size (see the
+ * conventions above); allocate stream buffers that will be read as
+ * homcomp_max_stream_bytes(nbEle) + HOMCOMP_STREAM_SLACK. */
+#define HOMCOMP_STREAM_SLACK 160
 /* The value the reference's wrappers store in *cmpSize for a stream of true length L. */
 size_t homcomp_ref_cmpsize(size_t stream_len, size_t nbEle);
 

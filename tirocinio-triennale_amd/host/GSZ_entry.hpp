@@ -155,7 +155,7 @@ inline void GSZ_compress_hostptr(float *oriData, unsigned char *cmpBytes, size_t
     const size_t cap = homcomp_max_stream_bytes(nbEle);
     int rc = HOMCOMP_OK;
     if (hipMalloc((void **)&d_ori, (nbEle ? nbEle : 1) * sizeof(float)) != hipSuccess ||
-        hipMalloc((void **)&d_cmp, cap ? cap : 1) != hipSuccess ||
+        hipMalloc((void **)&d_cmp, cap + HOMCOMP_STREAM_SLACK) != hipSuccess ||
         hipMemcpy(d_ori, oriData, nbEle * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
         rc = HOMCOMP_ERR_HIP;
     if (rc == HOMCOMP_OK) {
@@ -179,7 +179,7 @@ inline void GSZ_decompress_hostptr(float *decData, unsigned char *cmpBytes, size
     int rc = HOMCOMP_OK;
     if (cmpSize > cap) cmpSize = cap;
     if (hipMalloc((void **)&d_dec, (nbEle ? nbEle : 1) * sizeof(float)) != hipSuccess ||
-        hipMalloc((void **)&d_cmp, cap ? cap : 1) != hipSuccess ||
+        hipMalloc((void **)&d_cmp, cap + HOMCOMP_STREAM_SLACK) != hipSuccess ||
         hipMemset(d_cmp, 0, cap) != hipSuccess ||
         hipMemcpy(d_cmp, cmpBytes, cmpSize, hipMemcpyHostToDevice) != hipSuccess)
         rc = HOMCOMP_ERR_HIP;

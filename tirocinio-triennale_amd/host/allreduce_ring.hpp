@@ -113,9 +113,9 @@ public:
         release();
         stream_cap = homcomp_max_stream_bytes(max_block);
         bool ok = hipMalloc((void **)&d_rtmpbuf, (padded ? padded : 1) * sizeof(float)) == hipSuccess;
-        ok = ok && hipMalloc((void **)&d_cmpReduceBytes, stream_cap) == hipSuccess;
-        ok = ok && hipMalloc((void **)&d_inbuf[0], stream_cap) == hipSuccess;
-        ok = ok && hipMalloc((void **)&d_inbuf[1], stream_cap) == hipSuccess;
+        ok = ok && hipMalloc((void **)&d_cmpReduceBytes, stream_cap + HOMCOMP_STREAM_SLACK) == hipSuccess;
+        ok = ok && hipMalloc((void **)&d_inbuf[0], stream_cap + HOMCOMP_STREAM_SLACK) == hipSuccess;
+        ok = ok && hipMalloc((void **)&d_inbuf[1], stream_cap + HOMCOMP_STREAM_SLACK) == hipSuccess;
         if (int_deltas) ok = ok && hipMalloc((void **)&d_quant, (max_block ? max_block : 1) * sizeof(int)) == hipSuccess;
         if (!ok) {
             release();

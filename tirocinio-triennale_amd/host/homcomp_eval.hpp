@@ -258,8 +258,8 @@ inline EvalResult evaluate(const std::vector<float> &vec, const std::vector<floa
     bool ok = hipMalloc((void **)&d_vec, nbEle * sizeof(float)) == hipSuccess &&
               hipMalloc((void **)&d_local, nbEle * sizeof(float)) == hipSuccess &&
               hipMalloc((void **)&d_dec, nbEle * sizeof(float)) == hipSuccess &&
-              hipMalloc((void **)&d_minmax, 2 * sizeof(float)) == hipSuccess && hipMalloc((void **)&d_cmp, cap) == hipSuccess &&
-              hipMalloc((void **)&d_out, cap) == hipSuccess &&
+              hipMalloc((void **)&d_minmax, 2 * sizeof(float)) == hipSuccess && hipMalloc((void **)&d_cmp, cap + HOMCOMP_STREAM_SLACK) == hipSuccess &&
+              hipMalloc((void **)&d_out, cap + HOMCOMP_STREAM_SLACK) == hipSuccess &&
               hipMemcpy(d_vec, vec.data(), nbEle * sizeof(float), hipMemcpyHostToDevice) == hipSuccess &&
               hipMemcpy(d_local, vec_local.data(), nbEle * sizeof(float), hipMemcpyHostToDevice) == hipSuccess;
     if (!ok) {
