@@ -76,7 +76,8 @@ size_t homcomp_ref_cmpsize(size_t stream_len, size_t nbEle);
 
 /* Replaces the per-call cudaMalloc/cudaMemset/cudaFree of three (codec) or six (homomorphic
  * sum) scratch arrays in src/GSZ_entry.cu:275-280,519-530 -- the shape
- * allreduce_ring_comprs_hom_sum_F_opt hoists out of its loop (src/cuda_awareallreduce.cu:745-760). */
+ * allreduce_ring_comprs_hom_sum_F_opt hoists out of its loop (src/cuda_awareallreduce.cu:745-760).
+ * max_nbEle below about 8.79e12 (2^31 - 2^16 tiles of 4096 elements), else HOMCOMP_ERR_TOO_LARGE. */
 int homcomp_workspace_create(homcomp_workspace **ws, size_t max_nbEle);
 int homcomp_workspace_destroy(homcomp_workspace *ws);
 /* Tuning of a workspace; no counterpart in the reference, whose one-warp thread blocks wait for
