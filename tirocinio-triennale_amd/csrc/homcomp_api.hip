@@ -64,8 +64,9 @@ struct homcomp_workspace {
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint32_t out_slots;       // deferral depth of packed tiles (2..4); the device's spill area has this many slots per data wave
     bool holds_spill;         // counted among the users of the device's spill area
-    uint32_t sliced;          // bit-plane paths of the sums: HOMCOMP_SLICED=0 switches them off, 2 makes stream (+) local
-                              // operand take its own for every tile that allows it (1: where most tiles do)
+    uint32_t sliced;          // bit-plane paths of the sums: HOMCOMP_SLICED=0 switches them off; 1: chosen per call; 2: the
+                              // kernels with the path for few planes whatever the streams look like; 3: stream (+) stream
+                              // runs the kernel for wide blocks whatever the streams look like
     int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
 };
 
@@ -149,6 +150,7 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
 // fits a compute unit, which is slower than spilling: its largest slots are 7.3 KiB.)
 constexpr int kStageClasses = 3;
 constexpr uint64_t kBitplaneTileBytes = hc::kHostTileBlocks * 20u;
+constexpr uint64_t kWideTileBytes = hc::kHostTileBlocks * 24u;
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
     {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4112 + 64)},
@@ -309,7 +311,7 @@ int choose_stage_class(int op, uint64_t expected_tile_bytes, uint32_t out_slots)
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
     p.out_slots = ws->out_slots;
-    p.sliced = ws->sliced;
+    p.sliced = ws->sliced == 3u ? 1u : ws->sliced;
     if (op == hc::kOpDecompress) {
         p.stage_bytes = 0u;
         return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
@@ -326,6 +328,14 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
             p.sliced = (seen & 0xffffffffu) * 4u >= (uint64_t)p.n_tiles * 3u;
         else
             p.sliced = expected_tile_bytes <= kBitplaneTileBytes;
+    }
+    // stream (+) stream: the kernel for few planes (blocks of up to six go down its bit-plane
+    // path) or the one for wide blocks (up to 23), by the incoming bytes per tile
+    if (op == hc::kOpHomAdd) {
+        if (ws->sliced == 1u)
+            p.sliced = expected_tile_bytes <= kWideTileBytes ? 1u : 2u;
+        else if (ws->sliced != 0u)
+            p.sliced = ws->sliced == 3u ? 2u : 1u;
     }
     if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
     int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
@@ -521,7 +531,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
     ws->sliced = 1;
     if (const char *e = std::getenv("HOMCOMP_SLICED")) {
         const long v = std::strtol(e, nullptr, 10);
-        ws->sliced = v < 0 ? 0 : (v > 2 ? 2 : (int)v);
+        ws->sliced = v < 0 ? 0 : (v > 3 ? 3 : (int)v);
     }
     ws->spin_limit = kSpinLimit;
     if (const char *e = std::getenv("HOMCOMP_SPIN_LIMIT")) {

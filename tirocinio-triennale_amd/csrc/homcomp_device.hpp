@@ -693,6 +693,227 @@ __device__ __forceinline__ void sliced_write(lds_bytes stage, uint32_t pos, cons
         if (q < o.F) store_u32_any(stage + pos + o.ob + 4u + 4u * q, o.m[q]);
 }
 
+// ---------------------------------------------------------------- wide blocks in the bit-plane domain
+//
+// stream (+) stream for blocks of up to kWideMaxF planes, a block per lane as above, laid out
+// for many planes.  A lane reads its block from the sign word on in 16-byte pieces (word 0 of a
+// block's pieces is the sign word, word q + 1 is plane q; measured on MI355X, pieces at a
+// multiple of four bytes -- every block of a stream without outlier-mode blocks -- come in at
+// the rate of memory, words one by one at two thirds of it).  Only as many pieces as the widest
+// block of the wave needs are asked for, summed and written (`chunks`, wave-uniform), and a piece
+// is worked on as a whole: everything below is arranged by words of the block, not by planes.
+//
+// The sum works on sign and magnitude directly.  With d = sign_A ^ sign_B, a + (b ^ d) + d over
+// W planes is a + b where the signs agree (it fits: both are below 2^(W-1)) and a - b + 2^W where
+// they differ, whose carry out of plane W - 1 says a >= b; where it is missing the W planes are
+// negated (invert, ripple the +1) and the sign is B's.  A sum of zero has no sign
+// (HomComp/src/GSZ.cu:93: the sign bit is "delta < 0").
+//
+// Element 0 (bit 7 of every word) rides along like the others while both blocks are in plain
+// mode.  With an outlier-mode block in the pair its sum is made as a scalar beside the planes, as
+// in sliced_add, and bit 7 of the planes is left out.
+constexpr uint32_t kWideChunks = 6;
+constexpr uint32_t kWideWords = 4 * kWideChunks;      // the sign word and 23 planes
+// `chunks` pieces cover W = 4 * chunks - 1 planes, and the blocks summed over them have at most W - 1
+constexpr uint32_t kWideMaxF = kWideWords - 2;
+constexpr uint32_t kWideOutWords = kWideWords + 4;    // a sum has one plane more, and plain mode can take element 0 one plane further
+constexpr uint32_t kWideOutBytes = 8 + 4 * (kWideMaxF + 2);   // outlier bytes, sign word, planes
+
+// pieces from the sign word on that blocks of up to F planes are summed over
+__device__ __forceinline__ constexpr uint32_t wide_chunks_for(uint32_t F) { return (F + 1u) / 4u + 1u; }
+
+struct WideIn {
+    uint32_t first;           // the word at the block's start (the outlier bytes of an outlier-mode block)
+    uint32_t w[kWideWords];   // from the sign word on
+};
+
+struct WideOut {
+    uint32_t hdr, size, ob, F, a0, w[kWideOutWords];   // w[]: from the sign word on
+};
+
+// `rs` starts at the tile's payload and reaches 16 bytes beyond the last block that is read; a
+// block that is not to be read (digest 0) and the pieces beyond a block's planes ask for words
+// beyond every buffer and get zeros without touching memory.
+__device__ __forceinline__ void wide_request(__amdgpu_buffer_rsrc_t rs, uint32_t ofs, uint32_t digest, uint32_t chunks, WideIn &x)
+{
+    const uint32_t F = digest & 0x1fu, ob = digest >> 5;
+    const uint32_t base = digest ? ofs + ob : kSlicedNoRead;
+    x.first = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)(ob ? ofs : kSlicedNoRead), 0, 0);
+#pragma unroll
+    for (uint32_t j = 0; j < kWideChunks; ++j) {
+        if (j < chunks) {   // wave-uniform
+            const uint32_t at = 4u * j <= F ? base : kSlicedNoRead;   // word 4j is there when the block has 4j planes or more
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)at, (int)(16u * j), 0);
+            x.w[4 * j] = v.x;
+            x.w[4 * j + 1] = v.y;
+            x.w[4 * j + 2] = v.z;
+            x.w[4 * j + 3] = v.w;
+        } else {
+            x.w[4 * j] = x.w[4 * j + 1] = x.w[4 * j + 2] = x.w[4 * j + 3] = 0u;
+        }
+    }
+}
+
+// What the first part of a sum leaves for the second.
+struct WideSum {
+    uint32_t r[kWideWords];   // r[w], w >= 1: plane w - 1 of a + (b ^ d) + d
+    uint32_t neg;             // elements whose planes are still to be negated
+    uint32_t sign_a;          // A's sign word
+    uint32_t v0;              // blocks whose element 0 is summed beside the planes: that sum
+    uint32_t chunks;          // pieces the sum was made over (wave-uniform)
+    bool scalar0;
+};
+
+// delta_out = delta_A + delta_B for the lane's block, first part: the planes' sum.
+__device__ __forceinline__ void wide_sum(const WideIn &A, uint32_t digA, const WideIn &B, uint32_t digB, uint32_t chunks, WideSum &s)
+{
+    constexpr uint32_t E = 0x80u;   // element 0
+    const uint32_t FA = digA & 0x1fu, FB = digB & 0x1fu, obA = digA >> 5, obB = digB >> 5;
+    s.chunks = chunks;
+    s.scalar0 = (obA | obB) != 0u;   // element 0 is summed beside the planes
+    const uint32_t SA = A.w[0], SB = B.w[0];
+    s.sign_a = SA;
+    const uint32_t d = SA ^ SB;
+    uint32_t carry = d;
+#pragma unroll
+    for (uint32_t j = 0; j < kWideChunks; ++j) {
+        if (j < chunks) {   // wave-uniform
+#pragma unroll
+            for (uint32_t w = 4 * j ? 4 * j : 1; w < 4 * j + 4; ++w) {
+                // a word beyond the block's planes belongs to the next block
+                const uint32_t pa = w <= FA ? A.w[w] : 0u;
+                const uint32_t pb = w <= FB ? B.w[w] : 0u;
+                const uint32_t y = pb ^ d;
+                const uint32_t x = pa ^ y;
+                s.r[w] = x ^ carry;
+                carry = (x & carry) | (~x & pa);   // the majority of pa, y and carry
+            }
+        }
+    }
+    s.neg = d & ~carry;   // signs differ and a < b
+    // ---- element 0 beside the planes
+    s.v0 = 0u;
+    if (__builtin_amdgcn_ballot_w64(s.scalar0) != 0) {   // wave-uniform
+        // the magnitude of a plain-mode block's element 0 lies in its planes, an outlier-mode
+        // block's in the outlier (HomComp/src/GSZ.cu:913-917, 1005-1006)
+        uint32_t gA = 0, gB = 0;
+        if (__builtin_amdgcn_ballot_w64(s.scalar0 && (obA == 0u || obB == 0u)) != 0) {
+#pragma unroll
+            for (uint32_t j = 0; j < kWideChunks; ++j) {
+                if (j < chunks) {
+#pragma unroll
+                    for (uint32_t w = 4 * j ? 4 * j : 1; w < 4 * j + 4; ++w) {
+                        gA |= (w <= FA ? (A.w[w] >> 7) & 1u : 0u) << (w - 1);
+                        gB |= (w <= FB ? (B.w[w] >> 7) & 1u : 0u) << (w - 1);
+                    }
+                }
+            }
+        }
+        const uint32_t lowA = ~(0xffffff00u << ((8u * (obA - 1u)) & 31u)), lowB = ~(0xffffff00u << ((8u * (obB - 1u)) & 31u));
+        const uint32_t m0A = obA ? A.first & lowA : gA, m0B = obB ? B.first & lowB : gB;
+        const uint32_t v0A = (SA & E) ? 0u - m0A : m0A, v0B = (SB & E) ? 0u - m0B : m0B;
+        s.v0 = v0A + v0B;   // wrapping, as the reference's int
+    }
+}
+
+// Second part: magnitudes and signs of the sums, and the block's rate selection
+// (HomComp/src/GSZ.cu:151-167).
+__device__ __forceinline__ void wide_finish(const WideSum &s, WideOut &o)
+{
+    constexpr uint32_t E = 0x80u;   // element 0
+    const uint32_t chunks = s.chunks, neg = s.neg;
+    // ---- magnitudes, the planes in use, element 0's bits
+    uint32_t c = neg, any = 0, fr2 = 0, g = 0;
+#pragma unroll
+    for (uint32_t j = 0; j <= kWideChunks; ++j) {
+        if (j < chunks) {   // wave-uniform
+#pragma unroll
+            for (uint32_t w = 4 * j ? 4 * j : 1; w < 4 * j + 4; ++w) {
+                const uint32_t t = s.r[w] ^ neg;
+                const uint32_t m = t ^ c;
+                c &= t;
+                o.w[w] = m;
+                any |= m;
+                fr2 = (m & ~E) ? w : fr2;           // elements 1..31   (:153)
+                g |= ((m >> 7) & 1u) << (w - 1);
+            }
+        } else {
+            o.w[4 * j] = o.w[4 * j + 1] = o.w[4 * j + 2] = o.w[4 * j + 3] = 0u;
+        }
+    }
+    uint32_t sign = (s.sign_a ^ neg) & any;
+    // ---- element 0
+    uint32_t s0neg = sign & E;   // nonzero: the sum of element 0 is negative
+    o.a0 = g;
+    if (s.scalar0) {
+        const int32_t minus = (int32_t)(0u - s.v0);
+        o.a0 = (uint32_t)((int32_t)s.v0 > minus ? (int32_t)s.v0 : minus);   // |sum| (0x80000000 stays)
+        s0neg = (int32_t)s.v0 < 0 ? E : 0u;
+    }
+    o.w[0] = (sign & ~E) | s0neg;
+    // ---- rate selection
+    const uint32_t b0 = bit_num(o.a0);
+    uint32_t fr1 = b0 > fr2 ? b0 : fr2;                    // all 32 elements  (:152)
+    if (fr1 > 31u) fr1 = 31u;
+    const uint32_t ob = (b0 + 7u) >> 3;                    // :154
+    const uint32_t sz1 = fr1 ? 4u + 4u * fr1 : 0u;         // :156
+    const uint32_t sz2 = 4u + 4u * fr2 + ob;               // :157
+    const bool plain = sz1 <= sz2;                         // :158-164
+    o.hdr = plain ? fr1 : fr2 | 0x80u | ((ob - 1u) << 5);
+    o.size = plain ? sz1 : sz2;
+    o.F = plain ? fr1 : fr2;
+    o.ob = plain ? 0u : ob;
+    // bit 7 of the planes: element 0's bits in plain mode, clear in outlier mode.  They are in
+    // place where element 0 rode along; after a sum beside the planes they are put in.
+    const uint32_t keep = plain && !s.scalar0 ? ~0u : ~E;
+    if (__builtin_amdgcn_ballot_w64(keep != ~0u) != 0) {   // wave-uniform
+#pragma unroll
+        for (uint32_t j = 0; j < kWideChunks; ++j) {
+            if (j < chunks) {
+#pragma unroll
+                for (uint32_t w = 4 * j ? 4 * j : 1; w < 4 * j + 4; ++w) o.w[w] &= keep;
+            }
+        }
+    }
+    const uint32_t ins = plain && s.scalar0 ? o.a0 : 0u;
+    if (__builtin_amdgcn_ballot_w64(ins != 0u) != 0) {   // wave-uniform
+#pragma unroll
+        for (uint32_t j = 0; j <= kWideChunks; ++j) {
+            if (j <= chunks) {
+#pragma unroll
+                for (uint32_t w = 4 * j ? 4 * j : 1; w < 4 * j + 4; ++w) o.w[w] |= ((ins >> (w - 1)) & 1u) << 7;
+            }
+        }
+    }
+}
+
+typedef u32x4 __attribute__((aligned(1))) u32x4_unaligned;
+
+// The block's payload at `pos` of the stage: outlier bytes (a whole word is stored; what it
+// writes beyond them is overwritten by the sign word), sign word, planes.  The blocks of the
+// lanes that write together follow each other in the stage, and the words from the fourth on go
+// out in pieces of four, highest first: a block's last piece may reach up to 12 bytes into what
+// follows it, where the first words of the next blocks belong, and those are written after it
+// (by the last instructions here, or by the group of lanes that writes next).
+__device__ __forceinline__ void wide_write(lds_bytes stage, uint32_t pos, const WideOut &o, uint32_t chunks)
+{
+    if (o.hdr == 0u) return;
+    const lds_bytes at = stage + pos + o.ob;
+#pragma unroll
+    for (uint32_t j = kWideChunks; j >= 1; --j) {
+        if (j <= chunks) {   // wave-uniform
+            if (4u * j <= o.F)
+                *(__attribute__((address_space(3))) u32x4_unaligned *)(at + 16u * j) =
+                    u32x4{o.w[4 * j], o.w[4 * j + 1], o.w[4 * j + 2], o.w[4 * j + 3]};
+        }
+    }
+    if (o.ob) store_u32_any(stage + pos, o.a0);
+    store_u32_any(at, o.w[0]);
+#pragma unroll
+    for (uint32_t w = 1; w < 4; ++w)
+        if (w <= o.F) store_u32_any(at + 4u * w, o.w[w]);
+}
+
 // ---------------------------------------------------------------- output-offset scan
 //
 // The byte offset of a tile's payload in the outgoing stream is an exclusive prefix sum over

@@ -342,11 +342,14 @@ struct InRegs {
     u32x4 chunk;   // the lane's 16-byte chunk of a sub-step's payload range
 };
 
-// BITPLANE: the kernel has the bit-plane paths.  stream (+) local operand comes in both kinds: the
-// host launches the kind without them where the incoming streams are too wide for them anyway,
-// because the general path alone is the faster code for such data (fewer registers in use; a
-// tile of the general path costs about 8 % more in the kernel that has both).
-template <int NIN, int LOCAL, int OUT, bool BITPLANE>
+// BITPLANE: the kernel's bit-plane path (kPlanesNone: none).  stream (+) local operand comes with
+// and without the path for tiles of few planes: the host launches the kind without where the
+// incoming streams are too wide for it anyway, because the general path alone is the faster code
+// for such data (fewer registers in use; a tile of the general path costs about 8 % more in the
+// kernel that has both).  stream (+) stream comes with the path for few planes or with the one
+// for wide blocks.
+enum : int { kPlanesNone = 0, kPlanesFew = 1, kPlanesWide = 2 };
+template <int NIN, int LOCAL, int OUT, int BITPLANE>
 __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k_wave(const TileParams p)
 {
     constexpr bool kEnc = OUT == kOutStream;
@@ -363,10 +366,13 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     __shared__ __align__(4) uint8_t s_hdr_out[kW][kEnc ? kTileBlocks : 4];
     // one stage per wave: the incoming streams of a sub-step are decoded one after the other
     // stream (+) stream as a sum in the bit-plane domain, tile by tile where the tiles allow it
-    constexpr bool kSliced = BITPLANE && kEnc && NIN == 2 && LOCAL == kLocalNone;
+    constexpr bool kSliced = BITPLANE == kPlanesFew && kEnc && NIN == 2 && LOCAL == kLocalNone;
+    // the same for blocks of many planes
+    constexpr bool kWide = BITPLANE == kPlanesWide && kEnc && NIN == 2 && LOCAL == kLocalNone;
     // stream (+) local operand likewise, the local deltas turned into bit planes on the way
-    constexpr bool kSlicedLocal = BITPLANE && kEnc && NIN == 1 && LOCAL != kLocalNone;
-    constexpr bool kAnySliced = kSliced || kSlicedLocal;
+    constexpr bool kSlicedLocal = BITPLANE == kPlanesFew && kEnc && NIN == 1 && LOCAL != kLocalNone;
+    constexpr bool kAnySliced = kSliced || kSlicedLocal;   // the paths that keep a half tile's words in registers ahead of their use
+    constexpr bool kAnyPlanes = kAnySliced || kWide;
     // the planes of the local operand of half a tile, a row of 64 words per plane and one for the
     // deltas of the blocks' first elements; they share the wave's stage of incoming payload
     constexpr int kLocalRows = (int)kLocalFew + 1;
@@ -445,9 +451,9 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
                     const uint32_t d0 = z0 != 0u && o0 < room ? digests & 0xffu : 0u;
                     const uint32_t d1 = z1 != 0u && o1 < room ? digests >> 8 : 0u;
                     *reinterpret_cast<uint16_t *>(&s_hdr_in[wave][c][b][2 * lane]) = (uint16_t)(d0 | (d1 << 8));
-                    if constexpr (kAnySliced) {
-                        // stream (+) stream takes tiles of up to kSlicedMaxF planes, stream (+) local operand of up to kFewPlanes
-                        constexpr uint32_t most = kSliced ? kSlicedMaxF : kFewPlanes;
+                    if constexpr (kAnyPlanes) {
+                        // stream (+) stream takes tiles of up to kSlicedMaxF or kWideMaxF planes, stream (+) local operand of up to kFewPlanes
+                        constexpr uint32_t most = kWide ? kWideMaxF : (kSliced ? kSlicedMaxF : kFewPlanes);
                         const bool few = __builtin_amdgcn_ballot_w64((d0 & 0x1fu) > most || (d1 & 0x1fu) > most) == 0;
                         const uint32_t bit = 1u << b;
                         if (c == 0) few_ctx |= bit;
@@ -498,7 +504,7 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     };
     // (`wanted` false: nothing is read, the registers are only given a value)
     auto request_in = [&](int c, tidx r, int b, int s, InRegs (&in)[kIn], bool wanted = true) __attribute__((always_inline)) {
-        if constexpr (kSliced) {
+        if constexpr (kSliced || kWide) {
             if (!wanted) {   // wave-uniform; cheaper here than a request that fetches nothing
                 in[c].chunk = u32x4{0u, 0u, 0u, 0u};
                 return;
@@ -562,10 +568,11 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             }
         }
     };
-    // 32 blocks (outlier bytes, sign word, planes) must fit an empty slot: they are written at once
+    // the blocks written at once (outlier bytes, sign word, planes: 32 blocks, 16 wide ones) must fit an empty slot
     constexpr uint32_t kSlicedWords = kSlicedLocal ? kLocalFew + 1u : (uint32_t)kSlicedOutPlanes;
-    const bool sliced_ok = kAnySliced && p.sliced &&
-                           ((p.stage_bytes / p.out_slots) & ~15u) - 64u >= 32u * (8u + 4u * kSlicedWords) + 16u;
+    constexpr uint32_t kSlicedAtOnce = kWide ? 16u : 32u;
+    const bool sliced_ok = kAnyPlanes && p.sliced &&
+                           ((p.stage_bytes / p.out_slots) & ~15u) - 64u >= kSlicedAtOnce * (kWide ? kWideOutBytes : 8u + 4u * kSlicedWords) + 16u;
     // The local operand is only known to fit its planes (deltas within -8 .. 7) once it has been
     // quantised.  A tile goes down the bit-plane path when its incoming blocks have few planes
     // and the tile before gave no reason for doubt: a half tile whose local deltas did not fit is
@@ -581,8 +588,10 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     fetch_headers(0);
     prepare(0, 0);
     sliced_request_half(0, 0, sliced_ctx(0));
+    if constexpr (!kWide) {
 #pragma unroll
-    for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j], !sliced_ctx(0));
+        for (int j = 0; j < kDepth; ++j) request(0, 0, j, loc[j], in[j], !sliced_ctx(0));
+    }
 
     // Deferred tiles: a tile packed in round r is copied out in round r + D (D = p.out_slots, 2 to
     // 4): its total is published when it is packed, the prefix word is requested in round
@@ -861,6 +870,64 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
                     for (int j = 0; j < kDepth; ++j) request(r + 1, buf ^ 1, j, loc[j], in[j], !next_sliced);
                 }
+                if constexpr (kWide) {
+                    // ---- the whole tile in the bit-plane domain, 64 blocks (a block per lane) at a
+                    //      time: the blocks' words are asked for, in 16-byte pieces from the sign
+                    //      word on, as many as the widest block of the wave has; summed; written.
+                    //      Nothing travels ahead of its use here (the other waves of the SIMD
+                    //      fill the wait; registers for a half tile ahead are not to be had).
+#pragma unroll 1
+                    for (int half = 0; half < 2; ++half) {
+                        const int blk = half * 64 + lane;
+                        uint32_t dig[kIn], ofs[kIn];
+                        uint32_t widest = 0;
+#pragma unroll
+                        for (int c = 0; c < NIN; ++c) {
+                            dig[c] = (uint32_t)s_hdr_in[wave][c][buf][blk];
+                            ofs[c] = s_ofs_in[wave][c][buf][blk];
+                            widest = widest > (dig[c] & 0x1fu) ? widest : (dig[c] & 0x1fu);
+                        }
+                        uint32_t chunks = 1;
+#pragma unroll
+                        for (uint32_t j = 1; j < kWideChunks; ++j)
+                            if (__builtin_amdgcn_ballot_w64(wide_chunks_for(widest) > j) != 0) chunks = j + 1u;
+                        WideIn AB[kIn];
+#pragma unroll
+                        for (int c = 0; c < NIN; ++c) {
+                            const uint32_t room = buf ? room_ctx1[c] : room_ctx0[c];
+                            const uint32_t rel_end = buf ? end_ctx1[c] : end_ctx0[c];
+                            // a block that starts below the stated size is read in full (HomComp/src/GSZ.cu:908-911);
+                            // a block's last piece ends at most 12 bytes beyond the block
+                            uint32_t lim = room ? room + (kMaxBlockBytes - 1) + 16u : 0u;
+                            const uint32_t reach = rel_end + 16u;
+                            if (lim > reach) lim = reach;
+                            const __amdgpu_buffer_rsrc_t pay = buffer_of(p.in[c] + (buf ? start_ctx1[c] : start_ctx0[c]), lim);
+                            wide_request(pay, ofs[c], dig[c], chunks, AB[c]);
+                        }
+                        WideOut out;
+                        {
+                            WideSum sum;
+                            wide_sum(AB[0], dig[0], AB[kIn - 1], dig[kIn - 1], chunks, sum);
+                            wide_finish(sum, out);
+                        }
+                        s_hdr_out[wave][blk] = (uint8_t)out.hdr;
+                        const uint32_t incl = wave_incl_scan_u32(out.size, lane);
+                        // four writes of 16 blocks each, so that what is written at once fits an empty slot
+                        uint32_t before = 0;
+#pragma unroll 1
+                        for (int q = 0; q < 4; ++q) {
+                            const uint32_t upto = (uint32_t)__builtin_amdgcn_readlane((int)incl, 16 * q + 15);
+                            const uint32_t bytes = upto - before;
+                            make_room(bytes);   // always true here: 16 blocks fit an empty slot
+                            const uint32_t pos = run - flushed + (incl - out.size) - before;
+                            if ((lane >> 4) == q) wide_write((lds_bytes)stage, pos, out, chunks);
+                            run += bytes;
+                            before = upto;
+                        }
+                    }
+                    wave_lds_fence();
+                    prepare(r + 1, buf ^ 1);   // the next tile's block offsets
+                }
                 if constexpr (kSlicedLocal) {
                     // ---- stream (+) local operand in the bit-plane domain, half a tile at a time:
                     //      four sub-steps turn the local values into deltas (as the general path
@@ -946,6 +1013,18 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
                     for (int j = 0; j < kDepth; ++j) request_in(0, r + 1, buf ^ 1, j, in[j], !next_sliced);
                 }
+            } else if constexpr (kWide) {
+                // A tile with a block beyond the bit-plane path: the general path, its operands
+                // fetched on the spot.  (The host launches this kernel for streams whose tiles
+                // rarely come here, and nothing is kept in registers for them.)
+#pragma unroll 1
+                for (int s = 0; s < kSub; ++s) {
+                    SubRegs<LOCAL> now;
+                    InRegs now_in[kIn];
+                    request(r, buf, s, now, now_in);
+                    sub(s, now, now_in, r, buf, s, false);
+                }
+                prepare(r + 1, buf ^ 1);
             } else {
             planes_seen = 0;
 #pragma unroll 1
@@ -1237,7 +1316,7 @@ __global__ void k_fill_u64(uint64_t *p, uint64_t n)
 
 // ---------------------------------------------------------------- launchers
 
-template <int NIN, int LOCAL, int OUT, bool BITPLANE>
+template <int NIN, int LOCAL, int OUT, int BITPLANE>
 static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     // data workgroups of four waves (one tile per wave and round), on the encoder + the scan server
@@ -1250,7 +1329,7 @@ static hipError_t launch_wave(const TileParams &p, uint32_t max_grid, hipStream_
     return hipGetLastError();
 }
 
-template <int NIN, int LOCAL, int OUT, bool BITPLANE>
+template <int NIN, int LOCAL, int OUT, int BITPLANE>
 static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes, uint32_t max_stage_bytes)
 {
     const size_t dyn = OUT == kOutStream ? (size_t)(kWG / 64) * stage_bytes : 0;
@@ -1280,12 +1359,12 @@ static hipError_t wave_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes,
 }
 
 // both kinds of a kernel: the smaller of the two answers
-template <int NIN, int LOCAL, int OUT>
+template <int NIN, int LOCAL, int OUT, int A, int B>
 static hipError_t both_resident_blocks(int *blocks_per_cu, uint32_t stage_bytes, uint32_t max_stage_bytes)
 {
     int with = 0, without = 0;
-    hipError_t e = wave_resident_blocks<NIN, LOCAL, OUT, true>(&with, stage_bytes, max_stage_bytes);
-    if (e == hipSuccess) e = wave_resident_blocks<NIN, LOCAL, OUT, false>(&without, stage_bytes, max_stage_bytes);
+    hipError_t e = wave_resident_blocks<NIN, LOCAL, OUT, A>(&with, stage_bytes, max_stage_bytes);
+    if (e == hipSuccess) e = wave_resident_blocks<NIN, LOCAL, OUT, B>(&without, stage_bytes, max_stage_bytes);
     *blocks_per_cu = with < without ? with : without;
     return e;
 }
@@ -1294,11 +1373,11 @@ hipError_t op_kernel_residency(int op, uint32_t stage_bytes, uint32_t max_stage_
 {
     if (stage_bytes > max_stage_bytes) return hipErrorInvalidValue;
     switch (op) {
-    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream, false>(blocks_per_cu, stage_bytes, max_stage_bytes);
-    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32, false>(blocks_per_cu, stage_bytes, max_stage_bytes);
-    case kOpHomSumF32: return both_resident_blocks<1, kLocalF32, kOutStream>(blocks_per_cu, stage_bytes, max_stage_bytes);
-    case kOpHomSumI32: return both_resident_blocks<1, kLocalI32, kOutStream>(blocks_per_cu, stage_bytes, max_stage_bytes);
-    case kOpHomAdd: return wave_resident_blocks<2, kLocalNone, kOutStream, true>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpCompress: return wave_resident_blocks<0, kLocalF32, kOutStream, kPlanesNone>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpDecompress: return wave_resident_blocks<1, kLocalNone, kOutF32, kPlanesNone>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomSumF32: return both_resident_blocks<1, kLocalF32, kOutStream, kPlanesFew, kPlanesNone>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomSumI32: return both_resident_blocks<1, kLocalI32, kOutStream, kPlanesFew, kPlanesNone>(blocks_per_cu, stage_bytes, max_stage_bytes);
+    case kOpHomAdd: return both_resident_blocks<2, kLocalNone, kOutStream, kPlanesFew, kPlanesWide>(blocks_per_cu, stage_bytes, max_stage_bytes);
     default: return hipErrorInvalidValue;
     }
 }
@@ -1306,15 +1385,17 @@ hipError_t op_kernel_residency(int op, uint32_t stage_bytes, uint32_t max_stage_
 hipError_t launch_op(int op, const TileParams &p, uint32_t max_grid, hipStream_t s)
 {
     switch (op) {
-    case kOpCompress: return launch_wave<0, kLocalF32, kOutStream, false>(p, max_grid, s);
-    case kOpDecompress: return launch_wave<1, kLocalNone, kOutF32, false>(p, max_grid, s);
+    case kOpCompress: return launch_wave<0, kLocalF32, kOutStream, kPlanesNone>(p, max_grid, s);
+    case kOpDecompress: return launch_wave<1, kLocalNone, kOutF32, kPlanesNone>(p, max_grid, s);
     case kOpHomSumF32:
-        return p.sliced ? launch_wave<1, kLocalF32, kOutStream, true>(p, max_grid, s)
-                        : launch_wave<1, kLocalF32, kOutStream, false>(p, max_grid, s);
+        return p.sliced ? launch_wave<1, kLocalF32, kOutStream, kPlanesFew>(p, max_grid, s)
+                        : launch_wave<1, kLocalF32, kOutStream, kPlanesNone>(p, max_grid, s);
     case kOpHomSumI32:
-        return p.sliced ? launch_wave<1, kLocalI32, kOutStream, true>(p, max_grid, s)
-                        : launch_wave<1, kLocalI32, kOutStream, false>(p, max_grid, s);
-    case kOpHomAdd: return launch_wave<2, kLocalNone, kOutStream, true>(p, max_grid, s);
+        return p.sliced ? launch_wave<1, kLocalI32, kOutStream, kPlanesFew>(p, max_grid, s)
+                        : launch_wave<1, kLocalI32, kOutStream, kPlanesNone>(p, max_grid, s);
+    case kOpHomAdd:
+        return p.sliced == 2u ? launch_wave<2, kLocalNone, kOutStream, kPlanesWide>(p, max_grid, s)
+                              : launch_wave<2, kLocalNone, kOutStream, kPlanesFew>(p, max_grid, s);
     default: return hipErrorInvalidValue;
     }
 }

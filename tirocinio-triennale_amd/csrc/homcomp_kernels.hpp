@@ -37,8 +37,9 @@ struct TileParams {
     uint64_t *user_total;       // optional second destination for the stream length
     uint8_t *spill;             // out_slots slots of kSpillSlotBytes per data wave, for tiles that outgrow their LDS slot
     uint32_t out_slots;         // rounds a packed tile waits in LDS for its stream offset: 2 to 4
-    uint32_t sliced;            // the sums: tiles of few planes are summed in the bit-plane domain (0: never; stream (+) local
-                                // operand then runs the kernel without that path)
+    uint32_t sliced;            // the sums' bit-plane paths.  0: no tile takes one (stream (+) local operand then runs the
+                                // kernel without); 1: the kernel with the path for tiles of few planes; 2, stream (+)
+                                // stream only: the kernel with the path for wide blocks
     uint32_t plain;             // compress: the plain codec, every block in plain mode (0: the outlier codec)
     uint32_t stage_bytes;       // LDS bytes per data wave for those tiles (a multiple of 64); cut into out_slots slots
     uint64_t *host_total;       // optional pinned host word that also receives the stream length
