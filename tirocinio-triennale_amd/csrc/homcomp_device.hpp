@@ -731,26 +731,26 @@ struct WideOut {
     uint32_t hdr, size, ob, F, a0, w[kWideOutWords];   // w[]: from the sign word on
 };
 
-// `rs` starts at the tile's payload and reaches 16 bytes beyond the last block that is read; a
-// block that is not to be read (digest 0) and the pieces beyond a block's planes ask for words
-// beyond every buffer and get zeros without touching memory.
+// `rs` starts at the tile's payload and reaches 16 bytes beyond the last block that is read.
+// Only the lanes whose block has the piece take part in its load: a lane that asks for words
+// beyond the buffer gets zeros without a memory access, but costs the load unit as much as
+// one that reads (measured: the cache's access count was 2.4 times that of the words needed).
 __device__ __forceinline__ void wide_request(__amdgpu_buffer_rsrc_t rs, uint32_t ofs, uint32_t digest, uint32_t chunks, WideIn &x)
 {
     const uint32_t F = digest & 0x1fu, ob = digest >> 5;
-    const uint32_t base = digest ? ofs + ob : kSlicedNoRead;
-    x.first = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)(ob ? ofs : kSlicedNoRead), 0, 0);
+    x.first = 0u;
+    if (ob) x.first = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)ofs, 0, 0);
 #pragma unroll
     for (uint32_t j = 0; j < kWideChunks; ++j) {
+        u32x4 v = {0u, 0u, 0u, 0u};
         if (j < chunks) {   // wave-uniform
-            const uint32_t at = 4u * j <= F ? base : kSlicedNoRead;   // word 4j is there when the block has 4j planes or more
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)at, (int)(16u * j), 0);
-            x.w[4 * j] = v.x;
-            x.w[4 * j + 1] = v.y;
-            x.w[4 * j + 2] = v.z;
-            x.w[4 * j + 3] = v.w;
-        } else {
-            x.w[4 * j] = x.w[4 * j + 1] = x.w[4 * j + 2] = x.w[4 * j + 3] = 0u;
+            // word 4j is there when the block has 4j planes or more (a block that is not to be read has digest 0)
+            if (digest != 0u && 4u * j <= F) v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(ofs + ob), (int)(16u * j), 0);
         }
+        x.w[4 * j] = v.x;
+        x.w[4 * j + 1] = v.y;
+        x.w[4 * j + 2] = v.z;
+        x.w[4 * j + 3] = v.w;
     }
 }
 
