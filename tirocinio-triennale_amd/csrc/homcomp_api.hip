@@ -59,8 +59,10 @@ struct homcomp_workspace {
     uint32_t max_grid[hc::kOpCount][3];  // persistent grid of each operation's kernel, per LDS budget (small, medium, large)
     uint32_t full_grid[hc::kOpCount][3]; // the same at 100 percent (HOMCOMP_OPT_GRID_PERCENT scales it)
     uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
-    uint64_t *h_few;          // pinned host word, left by the offsets pre-pass of the last stream (+) local operand call that
-                              // got that far: n_tiles << 32 | tiles none of whose blocks has more than three planes
+    uint64_t *h_few;          // pinned host words, left by the offsets pre-pass of the last sum that got that far, n_tiles << 32 |
+                              // tiles that can take the bit-plane path for few planes: [0] stream (+) local operand (none of
+                              // the tile's blocks has more than three planes), [1] and [2] the two streams of stream (+)
+                              // stream (six)
     uint32_t spin_limit;      // bound on unsuccessful scan re-reads (HOMCOMP_SPIN_LIMIT overrides)
     uint32_t out_slots;       // deferral depth of packed tiles (2..4); the device's spill area has this many slots per data wave
     bool holds_spill;         // counted among the users of the device's spill area
@@ -114,7 +116,7 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
 
 // Offsets pre-pass of the incoming streams (header bytes -> payload offset of every tile): one
 // launch for all of them, under the epoch of the call's tile kernel.
-int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s, bool report_few = false)
+int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s)
 {
     hc::InOffsetsArgs a;
     std::memset(&a, 0, sizeof a);
@@ -135,7 +137,15 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
         a.block_words[c] = ws->d_in_blocks[c];
         a.ofs[c] = ws->d_in_ofs[c];
     }
-    if (report_few) a.few_report[0] = ws->h_few;
+    // the sums: how many tiles could take the bit-plane path for few planes (see run_tile_op)
+    if (p->local) {
+        a.few_report[0] = ws->h_few;
+        a.few_limit = hc::kFewPlanes;
+    } else if (n_streams == 2) {
+        a.few_report[0] = ws->h_few + 1;
+        a.few_report[1] = ws->h_few + 2;
+        a.few_limit = hc::kSlicedMaxF;
+    }
     return hip_ok(hc::launch_in_offsets(a, n_streams, p->n_tiles, p->hdr_bytes, epoch, ws->spin_limit, s)) ? HOMCOMP_OK
                                                                                                             : HOMCOMP_ERR_HIP;
 }
@@ -150,7 +160,7 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
 // fits a compute unit, which is slower than spilling: its largest slots are 7.3 KiB.)
 constexpr int kStageClasses = 3;
 constexpr uint64_t kBitplaneTileBytes = hc::kHostTileBlocks * 20u;
-constexpr uint64_t kWideTileBytes = hc::kHostTileBlocks * 24u;
+constexpr uint64_t kWideTileBytes = hc::kHostTileBlocks * 30u;   // blocks of six planes: 4 + 4 * 6 bytes and an outlier byte or two
 constexpr uint32_t kStage[kStageClasses][hc::kOpCount] = {
     {2 * (4096 + 64), 0, 2 * (3072 + 64), 2 * (3072 + 64), 2 * (2048 + 64)},
     {2 * (6464 + 64), 0, 2 * (4992 + 64), 2 * (4992 + 64), 2 * (4112 + 64)},
@@ -330,11 +340,18 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
             p.sliced = expected_tile_bytes <= kBitplaneTileBytes;
     }
     // stream (+) stream: the kernel for few planes (blocks of up to six go down its bit-plane
-    // path) or the one for wide blocks (up to 23), by the incoming bytes per tile
+    // path) or the one for wide blocks (up to 22): the first where most tiles can take its path
     if (op == hc::kOpHomAdd) {
-        if (ws->sliced == 1u)
-            p.sliced = expected_tile_bytes <= kWideTileBytes ? 1u : 2u;
-        else if (ws->sliced != 0u)
+        if (ws->sliced == 1u) {
+            // as above: by the previous call of the same length where there was one
+            const uint64_t seen_a = *(volatile const uint64_t *)(ws->h_few + 1), seen_b = *(volatile const uint64_t *)(ws->h_few + 2);
+            if (seen_a >> 32 == p.n_tiles && seen_b >> 32 == p.n_tiles) {
+                const uint64_t few = (seen_a & 0xffffffffu) < (seen_b & 0xffffffffu) ? (seen_a & 0xffffffffu) : (seen_b & 0xffffffffu);
+                p.sliced = few * 4u >= (uint64_t)p.n_tiles * 3u ? 1u : 2u;
+            } else {
+                p.sliced = expected_tile_bytes <= kWideTileBytes ? 1u : 2u;
+            }
+        } else if (ws->sliced != 0u)
             p.sliced = ws->sliced == 3u ? 2u : 1u;
     }
     if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
@@ -544,13 +561,13 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (v >= 0 && v <= (long)kMaxEpoch) ws->epoch = (uint32_t)v;
     }
     if (!ok || !hip_ok(hipMalloc(&ws->d_block, bytes)) || !hip_ok(hipMemset(ws->d_block, 0, bytes)) ||
-        !hip_ok(hipHostMalloc((void **)&ws->h_total, (3 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
+        !hip_ok(hipHostMalloc((void **)&ws->h_total, (5 + hc::kOpCount) * sizeof(uint64_t), hipHostMallocDefault))) {
         if (ws->d_block) (void)hipFree(ws->d_block);
         (void)spill_release(ws);
         delete ws;
         return HOMCOMP_ERR_HIP;
     }
-    std::memset(ws->h_total, 0, (3 + hc::kOpCount) * sizeof(uint64_t));
+    std::memset(ws->h_total, 0, (5 + hc::kOpCount) * sizeof(uint64_t));
     ws->h_mean_tile = ws->h_total + 2;
     ws->h_few = ws->h_mean_tile + hc::kOpCount;
     uint8_t *base = (uint8_t *)ws->d_block;
@@ -693,7 +710,7 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 1, &p, s, true))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
     return run_tile_op(ws, hc::kOpHomSumF32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 
@@ -714,7 +731,7 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     p.local = d_local_delta;
     p.out_cmp = d_cmp_out;
     p.user_total = d_stream_len;
-    if ((rc = in_offsets(ws, 1, &p, s, true))) return rc;
+    if ((rc = in_offsets(ws, 1, &p, s))) return rc;
     return run_tile_op(ws, hc::kOpHomSumI32, p, tile_bytes_of(p, cmp_in_size), s);
 }
 

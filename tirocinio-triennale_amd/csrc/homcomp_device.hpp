@@ -445,13 +445,12 @@ __device__ __forceinline__ void unpack8_add(const uint8_t *stage, uint32_t pos0,
 // 1005-1006), which has up to 32 bits.  In a word of the stream, byte k bit 7-m is element
 // 8k+m, so element 0 is bit 7; sums of deltas need no order of the elements, and the words go
 // out as they came in.
-constexpr uint32_t kSlicedMaxF = 6;
 constexpr int kSlicedOutPlanes = kSlicedMaxF + 2;   // plain mode can take element 0 one plane further
 // The common streams have one to three planes per block: code for kFewPlanes serves waves none
 // of whose blocks has more.  stream (+) local operand takes the bit-plane path for such tiles
 // only, with the local deltas as kLocalFew two's-complement planes (sign plane included), so a
 // sum has up to kLocalFew + 1 bits.
-constexpr uint32_t kFewPlanes = 3, kLocalFew = 4;
+constexpr uint32_t kLocalFew = 4;
 constexpr int kSlicedOutWords = kSlicedOutPlanes > (int)kLocalFew + 1 ? kSlicedOutPlanes : (int)kLocalFew + 1;
 
 typedef uint32_t __attribute__((aligned(1))) u32_unaligned;

@@ -1138,15 +1138,16 @@ __global__ __launch_bounds__(256) void k_in_offsets(const InOffsetsArgs a, uint3
         sum += dpp_u32<kDppXor1>(sum);
         sum += dpp_u32<kDppXor2>(sum);
         sum += dpp_u32<kDppRowHalfMirror>(sum);   // the other quad of the eight
-        // plane counts of the tile's blocks, or-ed: at most kFewPlanes if every one of them is
-        uint32_t planes = (q[it].x | q[it].y | q[it].z | q[it].w) & 0x1f1f1f1fu;
-        planes |= planes >> 16;
-        planes = (planes | (planes >> 8)) & 0x1fu;
-        planes |= dpp_u32<kDppXor1>(planes);
-        planes |= dpp_u32<kDppXor2>(planes);
-        planes |= dpp_u32<kDppRowHalfMirror>(planes);
+        // does any block of the tile have more than a.few_limit planes?  Byte-parallel: F + (127 -
+        // limit) reaches bit 7 of its byte exactly then (nothing carries from byte to byte)
+        const uint32_t slack = 0x7f7f7f7fu - a.few_limit * 0x01010101u;
+        uint32_t wider = (((q[it].x & 0x1f1f1f1fu) + slack) | ((q[it].y & 0x1f1f1f1fu) + slack) |
+                          ((q[it].z & 0x1f1f1f1fu) + slack) | ((q[it].w & 0x1f1f1f1fu) + slack)) & 0x80808080u;
+        wider |= dpp_u32<kDppXor1>(wider);
+        wider |= dpp_u32<kDppXor2>(wider);
+        wider |= dpp_u32<kDppRowHalfMirror>(wider);
         if ((threadIdx.x & (kPieces - 1)) == 0) {
-            if (tile < n_tiles) few_tiles += planes <= kFewPlanes ? 1u : 0u;
+            if (tile < n_tiles) few_tiles += wider == 0u ? 1u : 0u;
             s_tot[tile % kOfsBlockTiles] = sum;   // 0 beyond the last tile
         }
     }

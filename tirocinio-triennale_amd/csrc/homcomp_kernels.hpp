@@ -15,6 +15,9 @@ enum : int { kOpCompress = 0, kOpDecompress, kOpHomSumF32, kOpHomSumI32, kOpHomA
 constexpr uint32_t kHostTileElems = 4096;
 constexpr uint32_t kHostTileBlocks = kHostTileElems / 32u;
 constexpr uint32_t kHostChunkElems = 32768;
+// Plane counts the bit-plane paths of the sums take: stream (+) stream tiles none of whose blocks
+// has more than kSlicedMaxF (the kernel for few planes), stream (+) local operand kFewPlanes.
+constexpr uint32_t kSlicedMaxF = 6, kFewPlanes = 3;
 
 struct TileParams {
     const uint8_t *in[2];       // incoming streams (header + payload)
@@ -58,7 +61,8 @@ struct InOffsetsArgs {
     const uint8_t *hdr[2];      // the streams' header bytes
     uint64_t *block_words[2];   // per stream and block of 256 tiles: a word tagged with the launch's epoch, n_tiles / 256 + 1 of them
     uint64_t *ofs[2];           // result: absolute payload offset of every tile
-    uint64_t *few_report[2];    // optional (host-visible) word per stream: n_tiles << 32 | tiles none of whose blocks has more than three planes
+    uint64_t *few_report[2];    // optional (host-visible) word per stream: n_tiles << 32 | tiles none of whose blocks has more than few_limit planes
+    uint32_t few_limit;
     uint32_t *error;            // sticky error flags (bit 0: a bounded wait gave up)
 };
 // `epoch`: as TileParams::epoch, any value the block words have not seen since they were last cleared.
