@@ -508,6 +508,83 @@ def test_sum_kernel_follows_the_incoming_tiles(pkg, cuda, orc, gen, monkeypatch,
         g.close()
 
 
+@pytest.mark.parametrize("forced", [None, "2", "3"])
+def test_stream_plus_stream_wide_blocks(pkg, cuda, orc, monkeypatch, forced):
+    """stream (+) stream comes as two kernels: one whose bit-plane path takes tiles of at most six
+    planes and one that takes blocks of up to 22, a block per lane in 16-byte pieces, summed in
+    sign and magnitude (HOMCOMP_SLICED = 2 / 3 forces one; a workspace picks by the incoming bytes
+    per tile on its first call of a length and by the pre-pass's count of few-plane tiles of the
+    previous call afterwards).  Crafted deltas: every plane count 0..22 on both sides with both
+    signs (differences that change sign, carries into the 23rd and 24th plane), plain and outlier
+    mode on either side and in the result, outliers of 1..4 bytes, first elements and whole
+    blocks that cancel, tiles of empty blocks, blocks of 23..31 planes that send their tile
+    down the general path; payloads of random bytes under well-formed headers; unaligned
+    pointers; a stated size that cuts a stream short; wide and narrow calls in turn on one
+    workspace.  Every result must be the oracle's bytes."""
+    if forced is not None:
+        monkeypatch.setenv("HOMCOMP_SLICED", forced)
+    rng = np.random.default_rng(41)
+    n = 1 << 17
+    nb = n // 32
+
+    def craft(shift, top):
+        d = np.zeros((nb, 32), np.int64)
+        for b in range(nb):
+            F = int(rng.integers(0, top + 1))
+            if F:
+                d[b] = rng.integers(0, 1 << F, 32) * (rng.integers(0, 2, 32) * 2 - 1)
+                d[b, rng.integers(1, 32)] |= 1 << (F - 1)
+            kind = int(rng.integers(0, 7))
+            if kind == 0:      # outlier of 1..4 bytes in front
+                d[b, 0] = int(rng.integers(1, 1 << int(rng.integers(1, 32)))) * int(rng.integers(0, 2) * 2 - 1)
+            elif kind == 1:    # only the first element
+                d[b, 1:] = 0
+            elif kind == 2:    # empty block
+                d[b] = 0
+        at = (3 * 128 + shift) % nb
+        d[at:at + 128] = 0                                        # a tile of empty blocks
+        for t, F in enumerate(range(23, 32)):                     # wider than the path: general path for these tiles
+            d[(2 + 3 * t) * 128 + 17 + shift, 9] = (1 << (F - 1)) + 5
+        return d
+
+    def case(d1, d2, label):
+        d2 = d2.copy()
+        d2[::7, 0] = -d1[::7, 0]                                  # first elements that cancel
+        d2[1::11] = -d1[1::11]                                    # whole blocks that cancel
+        d2[2::13, 1:] = -d1[2::13, 1:] + np.sign(d1[2::13, 1:])   # differences of magnitude one, both signs
+        a, b = d1.reshape(-1).astype(np.int32), d2.reshape(-1).astype(np.int32)
+        s1, s2 = orc.encode_deltas(a), orc.encode_deltas(b)
+        total = a.astype(np.int64) + b.astype(np.int64)
+        want = orc.encode_deltas(((total + (1 << 31)) % (1 << 32) - (1 << 31)).astype(np.int32))
+        assert_stream_equal(orc.hom_add(s1, s2, n), want, f"oracle: hom_add of crafted streams ({label})")
+        return s1, s2, want
+
+    wide = case(craft(0, 22), craft(1, 22), "up to 22 planes")
+    narrow = case(craft(0, 6), craft(1, 6), "up to 6 planes")
+    mixed = case(craft(0, 22), craft(1, 6), "22 against 6")
+    g = Gpu(pkg, cuda, n)
+    try:
+        for step, (label, (s1, s2, want)) in enumerate([("wide", wide), ("wide", wide), ("narrow", narrow), ("narrow", narrow),
+                                                        ("mixed", mixed), ("wide", wide), ("narrow", narrow)]):
+            assert_stream_equal(g.hom_add(s1, s2, n), want, f"hom_add, call {step} ({label})")
+            assert_stream_equal(g.hom_add(s2, s1, n), want, f"hom_add, operands swapped, call {step} ({label})")
+        s1, s2, want = wide
+        assert_stream_equal(g.hom_add(s1, s2, n, offset=3), want, "hom_add, unaligned")
+        assert_stream_equal(g.hom_add(s1, s2, n, offset=1), want, "hom_add, unaligned by one")
+        hb = orc.header_bytes(n)
+        for cut in (hb + (s2.size - hb) // 2 + 5, hb + 1, s2.size - 3):
+            assert_stream_equal(g.hom_add(s1, s2, n, size_b=cut), orc.hom_add(s1, s2, n, size_b=cut), f"hom_add, second stream cut at {cut}")
+        # payloads of random bytes: sign bits on zero magnitudes, plane bits of element 0 in outlier mode
+        raw = []
+        for st in (s1, s2):
+            st = st.copy()
+            st[hb:] = rng.integers(0, 256, st.size - hb, dtype=np.uint8)
+            raw.append(st)
+        assert_stream_equal(g.hom_add(raw[0], raw[1], n), orc.hom_add(raw[0], raw[1], n), "hom_add of arbitrary payload bytes")
+    finally:
+        g.close()
+
+
 def test_two_streams_do_not_overlap_their_scans(pkg, cuda, orc, gen):
     """Two workspaces driven from two streams at the same time.  Every stream-producing kernel
     needs its whole grid resident, so the library orders such launches across the streams of a
