@@ -421,8 +421,17 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             if (t >= n_tiles) t = 0;   // loads are issued unconditionally; the values are not used then
 #pragma unroll
             for (int c = 0; c < NIN; ++c) {
-                const uint8_t *h = p.in[c] + (uint64_t)t * kTileBlocks + 2 * lane;
-                hdr_next[c] = (uint32_t)h[0] | ((uint32_t)h[1] << 8);
+                if constexpr (kSlicedLocal) {
+                    // Through a descriptor of the tile's header bytes: the address is the tile's, in
+                    // scalar registers, plus the lane.  These kernels use every vector register, and
+                    // the per-lane pointer the plain form keeps across the rounds was spilled to
+                    // scratch memory; fetching it back waits for every load under way (4 % of a call).
+                    const __amdgpu_buffer_rsrc_t hb = buffer_of(p.in[c] + (uint64_t)t * kTileBlocks, kTileBlocks);
+                    hdr_next[c] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(hb, 2 * lane, 0, 0);
+                } else {
+                    const uint8_t *h = p.in[c] + (uint64_t)t * kTileBlocks + 2 * lane;
+                    hdr_next[c] = (uint32_t)h[0] | ((uint32_t)h[1] << 8);
+                }
                 const uint64_t st = p.in_ofs[c][t];
                 start_next[c] = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(st >> 32)) << 32) |
                                 (uint32_t)__builtin_amdgcn_readfirstlane((int)st);
@@ -542,7 +551,11 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
     // kept alive through a tile of the general path)
     auto sliced_request_half = [&](int b, int half, bool wanted) __attribute__((always_inline)) {
         if constexpr (kAnySliced) {
-            const int blk = half * 64 + lane;
+            // (stream (+) local operand, see fetch_headers: the lane number taken anew, because the
+            // addresses made from it once and kept across the rounds were spilled to scratch memory)
+            int fresh_lane = lane;
+            if constexpr (kSlicedLocal) asm volatile("" : "+v"(fresh_lane));
+            const int blk = half * 64 + fresh_lane;
             bool more = false;
 #pragma unroll
             for (int c = 0; c < NIN; ++c) {
@@ -1043,9 +1056,16 @@ __global__ __launch_bounds__(kWG) __attribute__((amdgpu_waves_per_eu(4))) void k
             if constexpr (kEnc) {
                 wave_lds_fence();
                 // header bytes of the tile (HomComp/src/GSZ.cu:166)
+                if constexpr (kSlicedLocal) {   // (as for the incoming header bytes)
+                    const __amdgpu_buffer_rsrc_t ho = buffer_of(p.out_cmp + (uint64_t)t0 * kTileBlocks, kTileBlocks);
 #pragma unroll
-                for (int i = lane; i < kTileBlocks; i += 64)
-                    p.out_cmp[(uint64_t)t0 * kTileBlocks + i] = s_hdr_out[wave][i];
+                    for (int i = lane; i < kTileBlocks; i += 64)
+                        __builtin_amdgcn_raw_buffer_store_b8(s_hdr_out[wave][i], ho, i, 0, 0);
+                } else {
+#pragma unroll
+                    for (int i = lane; i < kTileBlocks; i += 64)
+                        p.out_cmp[(uint64_t)t0 * kTileBlocks + i] = s_hdr_out[wave][i];
+                }
                 if (lane == 0) scan_publish(scan, (uint32_t)t0, run);
             }
         }
