@@ -789,6 +789,11 @@ __device__ __forceinline__ void wide_sum(const WideIn &A, uint32_t digA, const W
             }
         }
     }
+    // (The carry is hidden from the compiler here.  The same sum written for the few-plane path
+    // came out wrong with hipcc 7.2 -- sums of zeros were 2^NP: the last plane, whose operands are
+    // constants, was folded into the three-input bit operations that follow -- and right with
+    // this empty statement in place, which costs nothing.)
+    asm("" : "+v"(carry));
     s.neg = d & ~carry;   // signs differ and a < b
     // ---- element 0 beside the planes
     s.v0 = 0u;
