@@ -58,7 +58,8 @@ struct homcomp_workspace {
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
     uint32_t max_grid[hc::kOpCount][3];  // persistent grid of each operation's kernel, per LDS budget (small, medium, large)
     uint32_t full_grid[hc::kOpCount][3]; // the same at 100 percent (HOMCOMP_OPT_GRID_PERCENT scales it)
-    uint64_t *h_mean_tile;    // pinned host words, one per operation: mean payload bytes per tile of its last finished call
+    uint64_t *h_mean_tile;    // pinned host words, one per operation, left by its last finished call: mean payload bytes per
+                              // tile and the share of tiles beyond a slot size asked about (TileParams::host_total)
     uint64_t *h_few;          // pinned host words, left by the offsets pre-pass of the last sum that got that far, n_tiles << 32 |
                               // tiles that can take the bit-plane path for few planes: [0] stream (+) local operand (none of
                               // the tile's blocks has more than three planes), [1] and [2] the two streams of stream (+)
@@ -354,8 +355,20 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         } else if (ws->sliced != 0u)
             p.sliced = ws->sliced == 3u ? 2u : 1u;
     }
-    if (expected_tile_bytes == 0) expected_tile_bytes = ws->h_mean_tile[op];   // 0 until a call has finished
+    const uint64_t seen = *(volatile const uint64_t *)&ws->h_mean_tile[op];   // 0 until a call has finished
+    if (expected_tile_bytes == 0) expected_tile_bytes = seen & 0xffffffffu;
     int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
+    // compress: the budget above holds the mean tile with an eighth to spare.  Tiles that vary
+    // (spikes in the data) do not need that: with half of them a little beyond the slots of the
+    // next smaller budget, that budget's extra workgroup per compute unit still wins (0.290
+    // against 0.314 ms on 1 GiB whose tiles average 6.4 KB, in 6.4 KB slots); with all of them
+    // beyond, it loses (0.394 against 0.308 ms).  So the kernel counts the tiles beyond that
+    // slot size, and the next call takes the smaller budget while they stay below 55 %.
+    if (op == hc::kOpCompress && cls > 0) {
+        const uint32_t smaller = kStage[cls - 1][op] / ws->out_slots - 64u;
+        p.probe_bytes = smaller & ~63u;
+        if (((seen >> 32) & 0xffffu) * 64u == p.probe_bytes && (seen >> 48) <= 140u) cls -= 1;
+    }
     if (ws->stage_class >= 0) cls = ws->stage_class;
     p.host_total = &ws->h_mean_tile[op];
     p.stage_bytes = kStage[cls][op];

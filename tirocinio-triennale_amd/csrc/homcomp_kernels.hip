@@ -95,6 +95,7 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
     // lane's place inside a step's words; lanes that take no part point beyond every array
     const uint32_t voff = (uint32_t)tid < lanes ? (uint32_t)tid * PER * 8u : 0xffffff00u;
     uint64_t base = 0;
+    uint32_t over = 0;   // the lane's tiles with more payload than p.probe_bytes
     auto words_from = [&](const uint64_t *arr, uint32_t t0) {
         // a window from the step's first word; capped below the offset of the lanes that stay out
         uint64_t left = t0 < c.n_tiles ? (uint64_t)(c.n_tiles - t0) * 8u : 0u;
@@ -186,6 +187,11 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
         }
         issue_order();
         base += step_total;
+        // (after the prefixes have gone out: the data waves wait for them)
+        if (p.probe_bytes != 0u) {
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j) over += v[j] > p.probe_bytes ? 1u : 0u;
+        }
     };
     // One loop shape for filling the pipeline and for the steady state: the first pass processes
     // two empty steps (a window beyond the end: no lane takes part) and issues the first two
@@ -207,12 +213,23 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
         process(at(t0 + step), 1, wb);
         request(at(t0 + 3ull * step), wb);
     }
+    // how many tiles were larger than the slot size the host asks about
+    __syncthreads();
+    const uint32_t over_wave = wave_incl_scan_u32(over, lane);
+    if (lane == 63) s_wave[0][wave] = over_wave;
+    __syncthreads();
     if (tid == 0) {
         const uint64_t len = p.hdr_bytes + base;   // HomComp/src/GSZ.cu:752-755
         *p.total = len;
         if (p.user_total) *p.user_total = len;
-        // mean payload bytes per tile, for the host's choice of the next launch's LDS budget
-        if (p.host_total) *p.host_total = base / c.n_tiles;
+        // for the host's choice of the next launch's LDS budget
+        if (p.host_total) {
+            uint32_t over_all = 0;
+#pragma unroll
+            for (int q = 0; q < kWG / 64; ++q) over_all += s_wave[0][q];
+            const uint64_t share = p.probe_bytes ? (uint64_t)over_all * 256u / c.n_tiles : 0u;
+            *p.host_total = ((base / c.n_tiles) & 0xffffffffu) | ((uint64_t)(p.probe_bytes / 64u) << 32) | (share << 48);
+        }
     }
 }
 

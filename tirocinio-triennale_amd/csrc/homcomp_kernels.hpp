@@ -45,7 +45,10 @@ struct TileParams {
                                 // stream only: the kernel with the path for wide blocks
     uint32_t plain;             // compress: the plain codec, every block in plain mode (0: the outlier codec)
     uint32_t stage_bytes;       // LDS bytes per data wave for those tiles (a multiple of 64); cut into out_slots slots
-    uint64_t *host_total;       // optional pinned host word that also receives the stream length
+    uint64_t *host_total;       // optional pinned host word for the host's choice of the next launch's LDS budget: mean payload
+                                // bytes per tile (bits 0-31), probe_bytes / 64 (bits 32-47), and how many of 256 tiles had more
+                                // payload than probe_bytes (bits 48-63)
+    uint32_t probe_bytes;       // a slot size the host would like to know that share for (0: none)
 };
 
 // Bytes per slot of the spill area (TileParams::spill): a whole worst-case tile.
