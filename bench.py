@@ -48,8 +48,10 @@ def measured_traffic(kind: str, log2n: int, rel: float):
     return None
 
 
-def time_op(torch, fn, iters: int) -> float:
-    """Average kernel-side milliseconds per call, HIP events on the launch stream."""
+def time_op(torch, fn, iters: int, warm: int = 0) -> float:
+    """Average kernel-side milliseconds per call, HIP events on the launch stream, after `warm` untimed calls."""
+    for _ in range(warm):
+        fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(iters):
@@ -203,8 +205,8 @@ def other_configs(torch, pkg, gen, orc):
         ws.compress(x, eb, ca)
         la = ws.last_size()
         e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3),
-             "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10), 4 * n + la),
-             "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(ca, la, n, eb, dec), 10), la + 4 * n)}
+             "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10, warm=2), 4 * n + la),
+             "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(ca, la, n, eb, dec), 10, warm=2), la + 4 * n)}
         if orc is not None:
             want = orc.compress(xh, np.float32(eb))
             ws.compress(x, eb, ca)
@@ -234,11 +236,11 @@ def other_configs(torch, pkg, gen, orc):
     ws.hom_sum_f32(ca, la, y, eb, cs)
     ls = ws.last_size()
     e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3), "compression_ratio_sum": round(4 * n / ls, 3),
-         "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 5), 4 * n + la),
-         "hom_sum_f32": op_entry(n, time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), 5), la + 4 * n + ls),
-         "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), 5), ls + 4 * n)}
+         "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 5, warm=2), 4 * n + la),
+         "hom_sum_f32": op_entry(n, time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), 5, warm=2), la + 4 * n + ls),
+         "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), 5, warm=2), ls + 4 * n)}
     ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8))   # dec doubles as the output buffer: 4N >= L here
-    e["hom_add"] = op_entry(n, time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8)), 5), la + lb + ls)
+    e["hom_add"] = op_entry(n, time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8)), 5, warm=2), la + lb + ls)
     ok = ws.last_size() == ls and bool(torch.equal(dec.view(torch.uint8)[:ls], cs[:ls]))
     e["hom_add_equals_hom_sum_f32"] = ok
     if orc is not None:
