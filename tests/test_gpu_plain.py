@@ -104,3 +104,40 @@ def test_plain_unaligned_and_saturated(gpu, orc):
         assert np.array_equal(got, want), first_diff(got, want)
         dec = gpu_decompress_plain(gpu, want, n, eb, offset=offset)
         assert np.array_equal(dec.view(np.uint32), orc.decompress_plain(want, n, eb).view(np.uint32))
+
+
+@pytest.mark.parametrize("kind,log2n,rel", [("uniform", 26, 1e-4), ("smooth", 26, 1e-6), ("gradient_like", 28, 1e-4),
+                                             ("uniform", 28, 1e-6)])
+def test_plain_codec_at_size(pkg, cuda, orc, gen, kind, log2n, rel):
+    """The plain codec at the sizes the benchmark runs (HomComp/src/GSZ.cu:1475-1991): stream and
+    reconstruction against the oracle on the same buffers, everything compared on the GPU."""
+    torch = cuda
+    orc.set_threads(16)
+    n = 1 << log2n
+    x = gen.GENERATORS_TORCH[kind](n, seed=4)
+    ws = pkg.Workspace(n)
+    try:
+        mm = torch.empty(2, dtype=torch.float32, device="cuda")
+        ws.value_range(x, mm)
+        r = mm.cpu().numpy()
+        eb = np.float32(pkg.rel_to_abs(rel, float(r[0]), float(r[1])))
+        cap = pkg.max_stream_bytes(n)
+        cmp = torch.full((cap + 160,), 0xA5, dtype=torch.uint8, device="cuda")
+        ws.compress_plain(x, float(eb), cmp)
+        L = ws.last_size()
+        xh = x.cpu().numpy()
+        want = orc.compress_plain(xh, eb)
+        assert L == want.size and torch.equal(cmp[:L], torch.from_numpy(want).cuda()), "plain stream differs from the oracle"
+        dec = torch.full((n,), 7.0, dtype=torch.float32, device="cuda")
+        ws.decompress_plain(cmp, n, float(eb), dec)
+        torch.cuda.synchronize()
+        want_dec = orc.decompress_plain(want, n, eb)
+        assert torch.equal(dec.view(torch.int32), torch.from_numpy(want_dec.view(np.int32)).cuda()), "plain reconstruction"
+        # the outlier decoder reads the plain stream to the same values
+        dec.fill_(7.0)
+        ws.decompress(cmp, L, n, float(eb), dec)
+        assert torch.equal(dec.view(torch.int32), torch.from_numpy(want_dec.view(np.int32)).cuda()), "outlier decoder on a plain stream"
+    finally:
+        ws.close()
+        del x
+        torch.cuda.empty_cache()

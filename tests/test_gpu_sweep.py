@@ -1,10 +1,11 @@
 """The size / kind / error-bound grid of the last benchmark configuration as a parity test:
-{smooth, gradient-like, uniform} x REL {1e-2, 1e-4, 1e-6} x 2^20, 2^22, 2^24 elements with
-compress, decompress, hom_sum_f32 and hom_add byte for byte against the CPU oracle, and at 2^26
-and 2^28 one bound per kind, again against the oracle (16 threads) on the very same buffers plus
-the size-independent properties of the codec (recompressing a reconstruction reproduces the
-stream; stream (+) floats and stream (+) stream meet in the same bytes; the sum decodes to the
-integer sum of the operands' quantised values).
+{smooth, gradient-like, uniform} x REL {1e-2, 1e-4, 1e-6} x 2^20 ... 2^28 elements (all 45 points)
+with compress, decompress, hom_sum_f32, quant_predict and hom_sum_i32 byte for byte against the
+CPU oracle (16 threads) on the very same buffers, hom_add against the oracle up to 2^26 and
+against hom_sum_f32's bytes at every size, plus the size-independent properties of the codec
+(recompressing a reconstruction reproduces the stream; stream (+) floats, stream (+) int32 deltas
+and stream (+) stream meet in the same bytes; the sum decodes to the integer sum of the
+operands' quantised values).
 """
 import numpy as np
 import pytest
@@ -52,7 +53,9 @@ class Point:
         assert ok, f"{what}: {first_diff(self.torch, got, want, got_len, want_np.size)}"
 
 
-def check_point(pt, full_oracle=True):
+def check_point(pt, full_oracle=True, properties=True):
+    """full_oracle: also the second operand's stream and hom_add against the oracle.  properties:
+    also the numpy passes over the quantised values (integer homomorphism, error bound)."""
     torch, ws, orc, n, eb = pt.torch, pt.ws, pt.orc, pt.n, pt.eb
     ca, cb, cs, cs2 = pt.buf(), pt.buf(), pt.buf(), pt.buf()
     ws.compress(pt.x, float(eb), ca)
@@ -74,18 +77,29 @@ def check_point(pt, full_oracle=True):
     pt.same(ca, la, want_a, "compress")
     want_s = orc.hom_sum_f32(want_a, yh, eb)
     pt.same(cs, ls, want_s, "hom_sum_f32")
+    # the Lorenzo pre-pass and the sum with its int32 deltas (HomComp/src/homcomp.cu:1553-1602, 1604-2921)
+    dlt = torch.full((n,), 12345, dtype=torch.int32, device="cuda")
+    pt.pkg.quant_predict(pt.y, float(eb), dlt)
+    ws.hom_sum_i32(ca, la, dlt, cs2)
+    li = ws.last_size()
+    want_d = orc.quant_predict(yh, eb)
+    assert torch.equal(dlt, torch.from_numpy(want_d).cuda()), "quant_predict"
+    assert li == ls and torch.equal(cs2[:li], cs[:ls]), "hom_sum_i32 and hom_sum_f32 differ"
+    del dlt, want_d
     if full_oracle:
         want_b = orc.compress(yh, eb)
         pt.same(cb, lb, want_b, "compress (second operand)")
         pt.same(cs2, ls2, orc.hom_add(want_a, want_b, n), "hom_add")
     want_dec = orc.decompress(want_s, n, eb)
     assert torch.equal(dec.view(torch.int32), torch.from_numpy(want_dec.view(np.int32)).cuda()), "decompressed sum"
-    # integer homomorphism and the error bound of a two-way sum
-    q = orc.decode_quants(want_s, n).astype(np.int64)
-    assert np.array_equal(q, orc.quantize_array(xh, eb).astype(np.int64) + orc.quantize_array(yh, eb)), "q(x)+q(y)"
-    exact = xh.astype(np.float64) + yh.astype(np.float64)
-    bound = 2 * float(eb) + 2.0 ** -20 * (np.abs(xh) + np.abs(yh)).astype(np.float64)
-    assert (np.abs(want_dec.astype(np.float64) - exact) <= bound).all(), "error bound of the sum"
+    if properties:
+        # integer homomorphism and the error bound of a two-way sum
+        q = orc.decode_quants(want_s, n).astype(np.int64)
+        assert np.array_equal(q, orc.quantize_array(xh, eb).astype(np.int64) + orc.quantize_array(yh, eb)), "q(x)+q(y)"
+        exact = xh.astype(np.float64) + yh.astype(np.float64)
+        bound = 2 * float(eb) + 2.0 ** -20 * (np.abs(xh) + np.abs(yh)).astype(np.float64)
+        assert (np.abs(want_dec.astype(np.float64) - exact) <= bound).all(), "error bound of the sum"
+        del q, exact, bound
     # recompressing the reconstruction of x reproduces its stream (|q| < 2^24 in every grid point)
     ws.decompress(ca, la, n, float(eb), dec)
     ws.compress(dec, float(eb), cs2)
@@ -106,10 +120,12 @@ def test_grid_against_oracle(pkg, orc, gen, cuda, kind, rel, log2n):
         pt.close()
 
 
-# one bound per kind at the two largest sizes: the bounds rotate so that every kind meets a coarse,
-# a medium and a fine bound across 2^26 and 2^28 together with the grid above
-LARGE = [("smooth", 26, 1e-6), ("gradient_like", 26, 1e-4), ("uniform", 26, 1e-2),
-         ("smooth", 28, 1e-2), ("gradient_like", 28, 1e-6), ("uniform", 28, 1e-4)]
+# Every kind and bound at the two largest sizes.  The numpy passes over the quantised values
+# (minutes of host time at 2^28) run at one bound per kind and size, rotated so that every kind
+# meets a coarse, a medium and a fine bound; the byte comparisons with the oracle run everywhere.
+WITH_PROPERTIES = {("smooth", 26, 1e-6), ("gradient_like", 26, 1e-4), ("uniform", 26, 1e-2),
+                   ("smooth", 28, 1e-2), ("gradient_like", 28, 1e-6), ("uniform", 28, 1e-4)}
+LARGE = [(kind, log2n, rel) for log2n in (26, 28) for kind in KINDS for rel in (1e-2, 1e-4, 1e-6)]
 
 
 @pytest.mark.parametrize("kind,log2n,rel", LARGE)
@@ -117,9 +133,10 @@ def test_large_sizes(pkg, orc, gen, cuda, kind, log2n, rel):
     orc.set_threads(16)
     pt = Point(pkg, cuda, gen, orc, kind, 1 << log2n, rel=rel)
     try:
-        check_point(pt, full_oracle=log2n < 28)
+        check_point(pt, full_oracle=log2n < 28, properties=(kind, log2n, rel) in WITH_PROPERTIES)
     finally:
         pt.close()
+        cuda.cuda.empty_cache()
 
 
 def test_config3_sums_on_wide_planes_1gib(pkg, orc, gen, cuda):
