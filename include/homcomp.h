@@ -111,7 +111,10 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
  * outlier codec), its payload the sign word and that many planes.  A plain stream is a stream
  * of the outlier codec whose blocks are all in plain mode: homcomp_decompress_f32 and the
  * homomorphic sums read it too.  The plain decoder has no out-of-bound rule (the reference's
- * kernel never looks at cmpSize): the buffer must hold the whole stream.  The reference's
+ * kernel never looks at cmpSize): every block the header bytes describe is read, so the buffer
+ * must hold the whole stream and be readable up to the 16-byte address boundary at or after its
+ * last byte (payload is fetched in aligned 16-byte pieces; nothing further out is touched, and the
+ * general rule about cmp_size + 160 above does not apply to this entry).  The reference's
  * wrapper reports a cmpSize that leaves out the payload of the last 32768-element chunk
  * (src/GSZ_entry.cu:176-180 reads the exclusive offset of the last thread block); the length
  * reported here is the true one. */
@@ -127,7 +130,10 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
                         uint64_t *d_stream_len, void *stream);
 
 /* homomorphic_sum (include/GSZ_entry.h:29-32, src/GSZ_entry.cu:456-502): the local operand is the
- * int32 output of homcomp_quant_predict_f32. */
+ * int32 output of homcomp_quant_predict_f32.  cmp_in_size is at most
+ * homcomp_ref_cmpsize(homcomp_max_stream_bytes(nbEle), nbEle), the largest value the reference's
+ * convention can state (HOMCOMP_ERR_INVALID_ARG beyond): a size stated as the capacity of a
+ * buffer laid out for a larger element count is not supported by this entry. */
 int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
                         const int32_t *d_local_delta, size_t nbEle, unsigned char *d_cmp_out,
                         uint64_t *d_stream_len, void *stream);

@@ -28,7 +28,7 @@ def closed_forms(ori32: np.ndarray, dec32: np.ndarray):
     big = np.abs(ori32) > 1
     with np.errstate(divide="ignore", invalid="ignore"):
         pw = np.where(big, (err32 / ori32).astype(np.float64), err)
-    mse = (err * err).mean()
+    mse = (err32 * err32).astype(np.float64).mean()     # squared in float32, summed in double (:112)
     do, dd = o - o.mean(), d - d.mean()
     return {"min": float(mn), "max": float(mx), "range": float(rng), "max_abs_err": float(err32.max()),
             "max_rel_err": float(np.float32(err32.max() / np.float32(mx - mn))),
@@ -64,18 +64,18 @@ def test_evaluator_report(tmp_path, orc, gen, cuda, kind, n, eb, rel):
     dec = orc.decompress(hs, n, eb_abs)
     got_dec = np.fromfile(out, np.float32)
     assert np.array_equal(got_dec.view(np.uint32), dec.view(np.uint32))
-    # every reported measure against its closed form.  As in the reference the comparison is
-    # against twice the first operand (float32), whatever the second operand was: with two
-    # different operands the measures then contain their difference, which exercises the formulas
-    # on large errors as well.
-    want = closed_forms(a * np.float32(2.0), dec)
+    # every reported measure against its closed form.  The reduced values are scored against the
+    # float32 sum of the two operands, which is the reference's "twice the input" (vec[i] *= 2,
+    # HomComp/src/homcomp_eval.cu:214-215) where the operands are one file, as in the first case.
+    want = closed_forms(a + b, dec)
+    if kind == "smooth":
+        assert np.array_equal(a + b, a * np.float32(2.0))
     for key in ("min", "max", "max_abs_err"):
         assert np.float32(kv[key]) == np.float32(want[key]), key
     for key in ("range", "max_rel_err", "max_pw_rel_err", "psnr", "nrmse", "correlation"):
         assert float(kv[key]) == pytest.approx(want[key], rel=1e-9, abs=1e-12), key
     assert float(kv["compression_ratio"]) == pytest.approx(4.0 * n / (hs.size + hb), rel=1e-12)
-    if kind == "smooth":
-        assert float(kv["max_abs_err"]) <= 2 * float(eb_abs) * (1 + 1e-3)
+    assert float(kv["max_abs_err"]) <= 2 * float(eb_abs) * (1 + 1e-3) + 2.0 ** -22 * float(np.abs(a + b).max())
     # the printed report carries the reference's wording
     for needle in ("Max absolute error =", "PSNR =", "acEff=", "Compression Ratio =", "HomComp_F speedup:"):
         assert needle in res.stdout

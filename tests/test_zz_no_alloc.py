@@ -89,3 +89,76 @@ def test_static_entry_limits_and_arguments(pkg, cuda):
     assert f(s.data_ptr(), 0, x.data_ptr(), 0, eb, s.data_ptr(), res.data_ptr(), None) == 0
     torch.cuda.synchronize()
     assert res.tolist() == [0, 0]
+
+
+def test_static_entry_allocates_nothing(pkg, cuda, orc, gen):
+    """The entry's one claim: after the first call on the device (which looks up the array's address
+    and the resident grid) a call changes neither the device's free memory nor torch's pools."""
+    torch = cuda
+    orc.set_threads(16)
+    n = 1 << 20
+    eb = np.float32(8e-4)
+    a, b = gen.smooth_np(n, 501), gen.smooth_np(n, 502)
+    sa = orc.compress(a, eb)
+    cap = pkg.max_stream_bytes(n)
+    buf = torch.zeros(cap + 160, dtype=torch.uint8, device="cuda")
+    buf[:sa.size] = torch.from_numpy(sa).cuda()
+    out = torch.zeros(cap + 160, dtype=torch.uint8, device="cuda")
+    res = torch.zeros(2, dtype=torch.int64, device="cuda")
+    dl = torch.from_numpy(b).cuda()
+    pkg.hom_sum_f32_static(buf, sa.size, dl, float(eb), out, res)       # first call: set-up allowed
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for smaller in (n, n // 4, n):                                     # the second with a smaller input
+        pkg.hom_sum_f32_static(buf, sa.size, dl[:smaller], float(eb), out, res, n=smaller)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_reserved() == reserved0
+    L, err = (int(v) for v in res.cpu())
+    want = orc.hom_sum_f32(sa, b, eb)
+    assert err == 0 and L == want.size and np.array_equal(out[:L].cpu().numpy(), want)
+
+
+def test_static_entry_in_a_graph(pkg, cuda, orc, gen):
+    """One static call recorded into a HIP graph after a warm-up call, replayed with new operands
+    and with eager calls of the same entry between the replays; every replay against the oracle."""
+    torch = cuda
+    orc.set_threads(16)
+    n = (1 << 19) + 32768
+    eb = np.float32(8e-4)
+    cap = pkg.max_stream_bytes(n)
+    buf = torch.zeros(cap + 160, dtype=torch.uint8, device="cuda")
+    out = torch.zeros(cap + 160, dtype=torch.uint8, device="cuda")
+    res = torch.zeros(2, dtype=torch.int64, device="cuda")
+    dl = torch.zeros(n, dtype=torch.float32, device="cuda")
+    eager_out = torch.zeros(cap + 160, dtype=torch.uint8, device="cuda")
+    eager_res = torch.zeros(2, dtype=torch.int64, device="cuda")
+
+    def load(seed):
+        a, b = gen.smooth_np(n, seed), gen.smooth_np(n, seed + 1)
+        sa = orc.compress(a, eb)
+        buf.fill_(0x5A)
+        buf[:sa.size] = torch.from_numpy(sa).cuda()
+        dl.copy_(torch.from_numpy(b).cuda())
+        return sa.size, orc.hom_sum_f32(sa, b, eb)
+
+    size, want = load(600)
+    pkg.hom_sum_f32_static(buf, cap, dl, float(eb), out, res)          # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        # the incoming size is stated as the capacity: the same graph serves streams of any length
+        pkg.hom_sum_f32_static(buf, cap, dl, float(eb), out, res)
+    for seed in (600, 610, 620):
+        size, want = load(seed)
+        out.fill_(0xA5)
+        graph.replay()
+        torch.cuda.synchronize()
+        L, err = (int(v) for v in res.cpu())
+        assert err == 0 and L == want.size and np.array_equal(out[:L].cpu().numpy(), want), f"replay with seed {seed}"
+        # the program's own eager work on the same scratch between the replays
+        pkg.hom_sum_f32_static(buf, size, dl[:1 << 16], float(eb), eager_out, eager_res, n=1 << 16)
+        torch.cuda.synchronize()
+        assert int(eager_res[1]) == 0
+    del graph

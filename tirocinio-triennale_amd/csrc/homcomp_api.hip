@@ -85,10 +85,28 @@ int check_ws(const homcomp_workspace *ws, size_t n)
     return HOMCOMP_OK;
 }
 
+bool stream_is_capturing(hipStream_t s)
+{
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;   // treated like a capture: nothing is executed eagerly on such a stream
+    }
+    return cap != hipStreamCaptureStatusNone;
+}
+
 // Fresh epoch for one launch; clears the scan words (the two arrays are adjacent) and the block
-// words of the offsets pre-pass when the 22-bit tag wraps.
+// words of the offsets pre-pass when the 22-bit tag wraps.  A launch that is being recorded into a
+// graph takes no epoch of the eager sequence: it runs under kGraphEpoch and its graph clears the
+// words it uses (chained_launch, in_offsets), and clears issued here would be recorded, not
+// executed, while the counter started over -- eager calls would then meet words tagged by calls
+// of four million launches ago.
 int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
 {
+    if (stream_is_capturing(s)) {
+        *epoch = kGraphEpoch;
+        return HOMCOMP_OK;
+    }
     if (ws->epoch >= kMaxEpoch) {
         const uint64_t blocks = (uint64_t)ws->max_tiles / 256 + 1;
         if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)) ||
@@ -123,10 +141,8 @@ int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStrea
     std::memset(&a, 0, sizeof a);
     a.error = ws->d_error;
     uint32_t epoch = p->epoch;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    if (stream_is_capturing(s)) {
         // as for the tile kernel (see chained_launch): a replay finds the words of the replay before
-        (void)hipGetLastError();
         epoch = kGraphEpoch;
         const uint64_t blocks = (uint64_t)p->n_tiles / 256 + 1;
         for (int c = 0; c < n_streams; ++c)
@@ -265,13 +281,11 @@ int spill_release(homcomp_workspace *ws)
 int chained_launch(int device, uint64_t *scan_words, uint64_t n_scan_words, int op, hc::TileParams p,
                    uint32_t max_grid, hipStream_t s)
 {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+    const bool capturing = stream_is_capturing(s);
     DeviceState &c = g_dev[device];
     std::lock_guard<std::mutex> lock(c.mu);
     if (!p.spill) p.spill = c.spill;
     if (capturing) {
-        (void)hipGetLastError();
         // A captured launch is replayed with the epoch it was captured with, so the scan words
         // of the previous replay would read as this call's: the graph clears them first (with
         // a kernel; memset nodes are avoided in graphs).
@@ -737,6 +751,9 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
     if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
     if (!d_cmp_in || !d_local_delta || !d_cmp_out) return HOMCOMP_ERR_INVALID_ARG;
     if (!aligned16(d_local_delta)) return HOMCOMP_ERR_ALIGNMENT;
+    // no stream of nbEle elements is longer than the first term, and callers of the reference state
+    // the length plus the header bytes (homcomp_ref_cmpsize); see the note at the declaration
+    if (cmp_in_size > homcomp_max_stream_bytes(nbEle) + homcomp_header_bytes(nbEle)) return HOMCOMP_ERR_INVALID_ARG;
     hc::TileParams p;
     if ((rc = fill_params(ws, nbEle, s, &p))) return rc;
     p.in[0] = d_cmp_in;
@@ -825,6 +842,9 @@ int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size
         !hip_ok(hc::launch_fill_u64(a.block_words[0], (uint64_t)p.n_tiles / 256 + 1, s)))
         return HOMCOMP_ERR_HIP;
     if (!hip_ok(hc::launch_in_offsets(a, 1, p.n_tiles, p.hdr_bytes, p.epoch, p.spin_limit, s))) return HOMCOMP_ERR_HIP;
+    // (Under capture chained_launch gives the tile kernel the graph's epoch while the pre-pass above
+    // ran under epoch 1.  The two need not agree: the tile kernel never reads the pre-pass's block
+    // words, only the plain offsets it leaves, and both kinds of words were cleared just above.)
     return chained_launch(device, nullptr, 0, hc::kOpHomSumF32, p, st->grid[cls], s);
 }
 

@@ -5,7 +5,8 @@
 // compress, the timed decompress + add + compress workflow, the timed homomorphic_sum_F on the same
 // operands, decompress, error measures of the reduced values against twice the input.
 //
-// Compile with hipcc (the header holds two small kernels).
+// Compile with hipcc (the header holds three small kernels; they have internal linkage, so the
+// header can be included in several translation units of a program).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -44,7 +45,7 @@ inline std::vector<float> read_binary_floats(const char *filename)
 }
 
 // HomComp/src/homcomp_eval.cu:47-55
-__global__ void sum2arrays(float *__restrict__ a, const float *b, size_t count)
+static __global__ void sum2arrays(float *__restrict__ a, const float *b, size_t count)
 {
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)blockDim.x * gridDim.x;
@@ -90,18 +91,24 @@ __device__ inline T block_fold(T v, F f, T *scratch)
     return r;
 }
 
-// `scale` multiplies the original values in float32 before they are compared (the evaluator
-// doubles its input, vec[i] *= 2, :214-215).
-__global__ __launch_bounds__(kEvalThreads) void k_eval_first(const float *ori, const float *dec, size_t n, float scale,
-                                                             EvalPartial *out)
+// The original value the reconstruction is compared with, in float32: ori[i] * scale (the
+// evaluator doubles its input, vec[i] *= 2, :214-215), or ori[i] + ori_b[i] when a second operand
+// is given (the same number where the operands coincide).
+__device__ inline float eval_original(const float *ori, const float *ori_b, size_t i, float scale)
+{
+    return ori_b ? ori[i] + ori_b[i] : ori[i] * scale;
+}
+
+static __global__ __launch_bounds__(kEvalThreads) void k_eval_first(const float *ori, const float *ori_b, const float *dec, size_t n,
+                                                                    float scale, EvalPartial *out)
 {
     __shared__ double s_d[kEvalThreads / 64];
     __shared__ float s_f[kEvalThreads / 64];
-    const float first = ori[0] * scale;
+    const float first = eval_original(ori, ori_b, 0, scale);
     double sum_ori = 0, sum_dec = 0, sum_err2 = 0, max_pw = 0;
     float mn = first, mx = first, diff = 0;
     for (size_t i = (size_t)blockIdx.x * kEvalThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kEvalThreads) {
-        const float o = ori[i] * scale, d = dec[i];
+        const float o = eval_original(ori, ori_b, i, scale), d = dec[i];
         sum_ori += o;
         sum_dec += d;
         if (mx < o) mx = o;
@@ -113,7 +120,7 @@ __global__ __launch_bounds__(kEvalThreads) void k_eval_first(const float *ori, c
             if (max_pw < rel) max_pw = rel;
         }
         if (diff < err) diff = err;
-        sum_err2 += (double)err * (double)err;
+        sum_err2 += (double)(err * err);   // squared in float32, then widened (:112: `sum += err * err` with a float err)
     }
     auto add = [](double a, double b) { return a + b; };
     auto dmax = [](double a, double b) { return a > b ? a : b; };
@@ -131,13 +138,13 @@ __global__ __launch_bounds__(kEvalThreads) void k_eval_first(const float *ori, c
     if (threadIdx.x == 0) out[blockIdx.x] = p;
 }
 
-__global__ __launch_bounds__(kEvalThreads) void k_eval_second(const float *ori, const float *dec, size_t n, float scale,
-                                                              double mean_ori, double mean_dec, EvalMoments *out)
+static __global__ __launch_bounds__(kEvalThreads) void k_eval_second(const float *ori, const float *ori_b, const float *dec, size_t n,
+                                                                     float scale, double mean_ori, double mean_dec, EvalMoments *out)
 {
     __shared__ double s_d[kEvalThreads / 64];
     double prod = 0, a2 = 0, b2 = 0;
     for (size_t i = (size_t)blockIdx.x * kEvalThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kEvalThreads) {
-        const double a = (double)(ori[i] * scale) - mean_ori, b = (double)dec[i] - mean_dec;
+        const double a = (double)eval_original(ori, ori_b, i, scale) - mean_ori, b = (double)dec[i] - mean_dec;
         prod += a * b;
         a2 += a * a;
         b2 += b * b;
@@ -153,11 +160,12 @@ __global__ __launch_bounds__(kEvalThreads) void k_eval_second(const float *ori, 
 }  // namespace detail
 
 // HomComp/src/homcomp_eval.cu:72-133 on device buffers: the original values are d_ori[i] * scale
-// (float32), the reconstruction d_dec; cmpSize as the reference's wrappers report it.  Two passes
-// as in the reference (means first, then the centred moments), accumulated in double.  Returns
-// false when a HIP call fails.
+// (float32), or d_ori[i] + d_ori_b[i] when d_ori_b is given; the reconstruction is d_dec; cmpSize
+// as the reference's wrappers report it.  Two passes as in the reference (means first, then the
+// centred moments), accumulated in double; the squared error is formed in float32 as the
+// reference forms it.  Returns false when a HIP call fails.
 inline bool error_evaluation(const float *d_ori, const float *d_dec, size_t nbEle, size_t cmpSize, ErrorStats *out,
-                             float scale = 1.0f, hipStream_t stream = 0)
+                             float scale = 1.0f, hipStream_t stream = 0, const float *d_ori_b = nullptr)
 {
     using namespace detail;
     if (nbEle == 0) return false;
@@ -169,7 +177,7 @@ inline bool error_evaluation(const float *d_ori, const float *d_dec, size_t nbEl
     const int blocks = (int)((nbEle + kEvalThreads - 1) / kEvalThreads < (size_t)kEvalBlocks ? (nbEle + kEvalThreads - 1) / kEvalThreads
                                                                                             : (size_t)kEvalBlocks);
     bool ok = true;
-    hipLaunchKernelGGL(k_eval_first, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_dec, nbEle, scale, (EvalPartial *)d_part);
+    hipLaunchKernelGGL(k_eval_first, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_ori_b, d_dec, nbEle, scale, (EvalPartial *)d_part);
     ok = ok && hipMemcpyAsync(part.data(), d_part, blocks * sizeof(EvalPartial), hipMemcpyDeviceToHost, stream) == hipSuccess &&
          hipStreamSynchronize(stream) == hipSuccess;
     double sum_ori = 0, sum_dec = 0, sum_err2 = 0, max_pw = 0;
@@ -185,7 +193,7 @@ inline bool error_evaluation(const float *d_ori, const float *d_dec, size_t nbEl
     }
     const double mean_ori = sum_ori / (double)nbEle, mean_dec = sum_dec / (double)nbEle;
     if (ok) {
-        hipLaunchKernelGGL(k_eval_second, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_dec, nbEle, scale, mean_ori, mean_dec,
+        hipLaunchKernelGGL(k_eval_second, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_ori_b, d_dec, nbEle, scale, mean_ori, mean_dec,
                            (EvalMoments *)d_part);
         ok = hipMemcpyAsync(mom.data(), d_part, blocks * sizeof(EvalMoments), hipMemcpyDeviceToHost, stream) == hipSuccess &&
              hipStreamSynchronize(stream) == hipSuccess;
@@ -236,7 +244,9 @@ struct EvalResult {
 
 // HomComp/src/homcomp_eval.cu:135-236 with both operands given (the reference reads the same file
 // twice).  rel: eb is relative to the value range of `vec` (:156-166; float32 arithmetic, done on
-// the device here).  The reduced values are left in d_dec_out when it is not null (nbEle floats).
+// the device here).  The reduced values are scored against vec[i] + vec_local[i] in float32, which
+// is the reference's vec[i] * 2 (:214-215) where the operands coincide.  The reduced values are
+// left in d_dec_out when it is not null (nbEle floats).
 inline EvalResult evaluate(const std::vector<float> &vec, const std::vector<float> &vec_local, float eb, bool rel,
                            float *d_dec_out = nullptr)
 {
@@ -311,8 +321,9 @@ inline EvalResult evaluate(const std::vector<float> &vec, const std::vector<floa
     if (last_status() != HOMCOMP_OK) return failed(last_status());
     res.cmpSize = cmpSize;
     res.cmpSizeSum = cmpSize2;
-    // :214-217: the reduced values against twice the input, CR from the sum's cmpSize
-    if (!error_evaluation(d_vec, d_dec, nbEle, cmpSize2, &res.stats, 2.0f)) return failed(HOMCOMP_ERR_HIP);
+    // :214-217: the reduced values against the sum of the operands (twice the input in the
+    // reference, whose operands are one file), CR from the sum's cmpSize
+    if (!error_evaluation(d_vec, d_dec, nbEle, cmpSize2, &res.stats, 1.0f, 0, d_local)) return failed(HOMCOMP_ERR_HIP);
     if (d_dec_out && hipMemcpy(d_dec_out, d_dec, nbEle * sizeof(float), hipMemcpyDeviceToDevice) != hipSuccess)
         return failed(HOMCOMP_ERR_HIP);
     release();
