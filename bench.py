@@ -179,7 +179,9 @@ def other_configs(torch, pkg, gen, orc):
                                       length read back to the host before the next call (what the
                                       reference's ring does with MPI_Get_count) and once without any
                                       host round trip (the incoming size is stated as the buffer capacity,
-                                      the lengths stay in device words)
+                                      the lengths stay in device words); every call leaves the tile
+                                      offsets of its stream beside it and the next one takes them from
+                                      there instead of scanning the header bytes (also timed without)
     """
     import numpy as np
     res = {}
@@ -266,39 +268,51 @@ def other_configs(torch, pkg, gen, orc):
     ws.close()
     ws = pkg.Workspace(chunk)
     cap = pkg.max_stream_bytes(chunk)
-    cur = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
-    nxt = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    cur = [torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
+    nxt = [torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda") for _ in range(ranks)]
     lens = torch.zeros(ranks, dtype=torch.int64, device="cuda")
+    # tile offsets beside every chunk's stream (8 bytes per 4096 elements: they travel with the chunk)
+    tiles = pkg.tile_offsets_count(chunk)
+    ofs_cur = [torch.zeros(tiles, dtype=torch.int64, device="cuda") for _ in range(ranks)]
+    ofs_nxt = [torch.zeros(tiles, dtype=torch.int64, device="cuda") for _ in range(ranks)]
 
-    def ring(read_back: bool):
+    def ring(read_back: bool, offsets: bool = True):
         a, b = cur, nxt
+        oa, ob = ofs_cur, ofs_nxt
         sizes = [cap] * ranks
         for c in range(ranks):
+            if offsets:
+                ws.tile_offsets(out=oa[c])
             ws.compress(data[c][c * chunk:(c + 1) * chunk], eb, a[c], stream_len=lens[c:c + 1])
             if read_back:
                 sizes[c] = ws.last_size()
         for k in range(1, ranks):
             for c in range(ranks):
+                if offsets:
+                    ws.tile_offsets(in_a=oa[c], out=ob[c])
                 ws.hom_sum_f32(a[c], sizes[c], data[(c + k) % ranks][c * chunk:(c + 1) * chunk], eb, b[c],
                                stream_len=lens[c:c + 1])
                 if read_back:
                     sizes[c] = ws.last_size()
             a, b = b, a
+            oa, ob = ob, oa
         return a
 
-    def timed(read_back: bool):
-        ring(read_back)
+    def timed(read_back: bool, offsets: bool = True):
+        ring(read_back, offsets)
         torch.cuda.synchronize()
         best = float("inf")
         for _ in range(3):
             t0 = time.perf_counter()
-            final = ring(read_back)
+            final = ring(read_back, offsets)
             torch.cuda.synchronize()
             best = min(best, time.perf_counter() - t0)
         return best * 1e3, final
 
     ms_dev, final = timed(False)
     final_lens = [int(v) for v in lens.cpu()]
+    ms_dev_prepass, final_p = timed(False, offsets=False)
+    prepass_same = all(bool(torch.equal(final[c][:final_lens[c]], final_p[c][:final_lens[c]])) for c in range(ranks))
     ms_host, final_h = timed(True)
     # the schedule without host round trips recorded into one HIP graph (no call allocates or blocks)
     ms_graph, graph_same = None, None
@@ -322,14 +336,15 @@ def other_configs(torch, pkg, gen, orc):
     except Exception as exc:   # the figure is an extra; the eager schedules above stand without it
         print(f"ring graph replay skipped: {exc!r}", file=sys.stderr)
     e = {"ranks": ranks, "elements_per_rank": n_rank, "chunk_elements": chunk, "eb_abs": eb, "calls": "8 compress + 56 hom_sum_f32",
-         "ms_lengths_on_device": round(ms_dev, 4), "ms_lengths_read_back": round(ms_host, 4),
+         "ms_lengths_on_device": round(ms_dev, 4), "ms_lengths_on_device_without_tile_offsets": round(ms_dev_prepass, 4),
+         "ms_lengths_read_back": round(ms_host, 4),
          "GBps_rank_data_lengths_on_device": round(ranks * 4 * n_rank / ms_dev / 1e6, 1),
          "GBps_rank_data_lengths_read_back": round(ranks * 4 * n_rank / ms_host / 1e6, 1),
          "compression_ratio_reduced": round(ranks * 4 * chunk / sum(final_lens), 3)}
     if ms_graph is not None:
         e["ms_lengths_on_device_graph_replay"] = round(ms_graph, 4)
         e["graph_replay_same_bytes"] = graph_same
-    ok = all(bool(torch.equal(final[c][:final_lens[c]], final_h[c][:final_lens[c]])) for c in range(ranks))
+    ok = prepass_same and all(bool(torch.equal(final[c][:final_lens[c]], final_h[c][:final_lens[c]])) for c in range(ranks))
     e["both_modes_same_bytes"] = ok
     if orc is not None:
         # the oracle's chain for one chunk, and integer addition of the ranks' quantised values for it

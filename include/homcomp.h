@@ -93,6 +93,27 @@ int homcomp_workspace_destroy(homcomp_workspace *ws);
 #define HOMCOMP_OPT_SPIN_LIMIT 2
 int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value);
 
+/* Tile offsets: a side array that spares the call that reads a stream its pass over the header
+ * bytes.  The payload position of a block follows from the header bytes of all blocks before it
+ * (src/GSZ.cu:790-874 sums them per 32768-element chunk and scans the sums in the same kernel); a
+ * call here does that in a launch of its own ahead of the tile kernel, about 5 us for a stream of
+ * any length up to 4M elements -- a third of a ring step's call.  The call that PRODUCES a stream
+ * knows the offsets already, so it can leave them in a caller buffer, and the call that reads the
+ * stream can take them from there:
+ *   entry t (uint64, t < homcomp_tile_offsets_count(nbEle)) = byte offset, from the start of the
+ *   stream, of the payload of elements 4096 t .. 4096 t + 4095 (header bytes included; entry 0 is
+ *   homcomp_header_bytes(nbEle)).
+ * The array is a function of the stream's header bytes alone.  In a ring it travels with the
+ * chunk (8 bytes per 4096 elements: 8 KB beside a 4M-element chunk).
+ * homcomp_workspace_tile_offsets hands arrays over for the NEXT call on ws that reads or produces
+ * a stream, and that call only: d_in_a / d_in_b for its first / second incoming stream (NULL: the
+ * call computes them as usual), d_out (NULL: none) receives the offsets of the stream it produces.
+ * Device pointers, 16-byte aligned, homcomp_tile_offsets_count(nbEle) entries.  Offsets that do not
+ * belong to the stream give wrong values, never accesses beyond the stream's stated size.  No
+ * counterpart in the reference. */
+size_t homcomp_tile_offsets_count(size_t nbEle);
+int homcomp_workspace_tile_offsets(homcomp_workspace *ws, const uint64_t *d_in_a, const uint64_t *d_in_b, uint64_t *d_out);
+
 /* GSZ_compress_deviceptr_outlier (include/GSZ_entry.h:14-16, src/GSZ_entry.cu:263-301).
  * d_stream_len (optional, device uint64) receives L when the kernel finishes. */
 int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEle, float eb,

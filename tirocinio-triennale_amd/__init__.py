@@ -18,7 +18,8 @@ LIB_PATH = os.path.join(_HERE, "libhomcomp_amd.so")
 EXPORTS = (
     "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
     "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
-    "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_compress_f32", "homcomp_decompress_f32",
+    "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_tile_offsets_count",
+    "homcomp_workspace_tile_offsets", "homcomp_compress_f32", "homcomp_decompress_f32",
     "homcomp_compress_plain_f32", "homcomp_decompress_plain_f32",
     "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add", "homcomp_hom_sum_f32_static",
     "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
@@ -65,6 +66,9 @@ def lib() -> C.CDLL:
         L.homcomp_workspace_create.argtypes = [C.POINTER(vp), sz]
         L.homcomp_workspace_destroy.argtypes = [vp]
         L.homcomp_workspace_set_option.argtypes = [vp, C.c_int, C.c_long]
+        L.homcomp_tile_offsets_count.argtypes = [sz]
+        L.homcomp_tile_offsets_count.restype = sz
+        L.homcomp_workspace_tile_offsets.argtypes = [vp, vp, vp, vp]
         L.homcomp_compress_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_decompress_f32.argtypes = [vp, vp, sz, sz, C.c_float, vp, vp]
         L.homcomp_compress_plain_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
@@ -92,6 +96,13 @@ def header_bytes(n: int) -> int:
 
 def max_stream_bytes(n: int) -> int:
     return int(lib().homcomp_max_stream_bytes(n))
+
+
+def tile_offsets_count(n: int) -> int:
+    return int(lib().homcomp_tile_offsets_count(n))
+
+
+STREAM_SLACK = 160   # HOMCOMP_STREAM_SLACK: bytes an input stream buffer must be readable beyond its stated size
 
 
 def ref_cmpsize(stream_len: int, n: int) -> int:
@@ -132,6 +143,13 @@ class Workspace:
 
     def set_option(self, option: int, value: int) -> None:
         _check(lib().homcomp_workspace_set_option(self._h, int(option), int(value)), "workspace_set_option")
+
+    def tile_offsets(self, in_a=None, in_b=None, out=None) -> None:
+        """Tile offsets for the next call on this workspace (homcomp_workspace_tile_offsets): int64 device
+        tensors of tile_offsets_count(n) entries; the incoming streams' as left by the calls that
+        produced them, and/or where the next call leaves those of the stream it produces."""
+        ptr = lambda t: None if t is None else t.data_ptr()
+        _check(lib().homcomp_workspace_tile_offsets(self._h, ptr(in_a), ptr(in_b), ptr(out)), "workspace_tile_offsets")
 
     def __del__(self):
         try:

@@ -17,11 +17,15 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 
-// Epochs 1 .. kMaxEpoch go to eager launches in turn; kGraphEpoch is kept for launches recorded
-// into a graph, which are replayed with the epoch they were captured with and clear the scan
-// words first: an eager call is never handed the epoch whose words a replay left behind.
-constexpr uint32_t kGraphEpoch = (1u << 22) - 1;
-constexpr uint32_t kMaxEpoch = kGraphEpoch - 1;
+// Epochs 1 .. kMaxEpoch go to eager launches in turn.  The epochs above them are kept for launches
+// recorded into a graph, which are replayed with the epoch they were captured with: the first
+// launch a capture records on a workspace is preceded by kernels that clear the workspace's tagged
+// words, the launches of that capture take the graph epochs in turn (the clears are recorded again
+// when they run out), so a replay starts from cleared words and no call inside it meets the words
+// of another, and an eager call is never handed an epoch whose words a replay left behind.
+constexpr uint32_t kGraphEpochLast = (1u << 22) - 1;
+constexpr uint32_t kGraphEpochFirst = kGraphEpochLast - 4095;
+constexpr uint32_t kMaxEpoch = kGraphEpochFirst - 1;
 // Unsuccessful scan re-reads before a wave gives up (each costs a memory round trip, so this is
 // some tens of milliseconds): long enough for any delay of a resident workgroup, short enough
 // that a launch which could not become resident ends with an error instead of stalling for minutes.
@@ -56,6 +60,11 @@ struct homcomp_workspace {
     float *d_partial;         // min/max partials
     uint64_t *h_total;        // pinned host words (length, error) for the blocking read-back
     uint32_t epoch;           // last epoch handed out (1..kMaxEpoch)
+    unsigned long long capture_id;   // the stream capture whose launches take graph epochs at the moment (0: none yet)
+    uint32_t graph_epoch;     // the next of them
+    // Tile offsets handed over for the next call (homcomp_workspace_tile_offsets), cleared by it
+    const uint64_t *next_in_ofs[2];
+    uint64_t *next_out_ofs;
     uint32_t max_grid[hc::kOpCount][3];  // persistent grid of each operation's kernel, per LDS budget (small, medium, large)
     uint32_t full_grid[hc::kOpCount][3]; // the same at 100 percent (HOMCOMP_OPT_GRID_PERCENT scales it)
     uint64_t *h_mean_tile;    // pinned host words, one per operation, left by its last finished call: mean payload bytes per
@@ -75,6 +84,18 @@ struct homcomp_workspace {
 
 namespace {
 
+// The tile offsets handed over for a call are that call's only, however it ends.
+struct HandOver {
+    homcomp_workspace *ws;
+    explicit HandOver(homcomp_workspace *w) : ws(w) {}
+    ~HandOver()
+    {
+        if (!ws) return;
+        ws->next_out_ofs = nullptr;
+        ws->next_in_ofs[0] = ws->next_in_ofs[1] = nullptr;
+    }
+};
+
 int check_ws(const homcomp_workspace *ws, size_t n)
 {
     if (!ws) return HOMCOMP_ERR_INVALID_ARG;
@@ -85,34 +106,53 @@ int check_ws(const homcomp_workspace *ws, size_t n)
     return HOMCOMP_OK;
 }
 
-bool stream_is_capturing(hipStream_t s)
+// `id`: the capture's identifier (unique per capture), 0 outside a capture.
+bool stream_is_capturing(hipStream_t s, unsigned long long *id = nullptr)
 {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+    unsigned long long cid = 0;
+    if (hipStreamGetCaptureInfo(s, &cap, &cid) != hipSuccess) {
         (void)hipGetLastError();
-        return true;   // treated like a capture: nothing is executed eagerly on such a stream
+        cap = hipStreamCaptureStatusInvalidated;   // treated like a capture: nothing is executed eagerly on such a stream
+        cid = ~0ull;
     }
+    if (id) *id = cap != hipStreamCaptureStatusNone ? (cid ? cid : ~0ull) : 0;
     return cap != hipStreamCaptureStatusNone;
+}
+
+int clear_tagged_words(homcomp_workspace *ws, hipStream_t s)
+{
+    const uint64_t blocks = (uint64_t)ws->max_tiles / 256 + 1;
+    return hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)) &&
+                   hip_ok(hc::launch_fill_u64(ws->d_in_blocks[0], blocks, s)) &&
+                   hip_ok(hc::launch_fill_u64(ws->d_in_blocks[1], blocks, s))
+               ? HOMCOMP_OK
+               : HOMCOMP_ERR_HIP;
 }
 
 // Fresh epoch for one launch; clears the scan words (the two arrays are adjacent) and the block
 // words of the offsets pre-pass when the 22-bit tag wraps.  A launch that is being recorded into a
-// graph takes no epoch of the eager sequence: it runs under kGraphEpoch and its graph clears the
-// words it uses (chained_launch, in_offsets), and clears issued here would be recorded, not
-// executed, while the counter started over -- eager calls would then meet words tagged by calls
-// of four million launches ago.
+// graph takes no epoch of the eager sequence (clears issued for it are recorded, not executed, so
+// the eager counter must not start over on their account): it takes the next graph epoch, and the
+// first launch of a capture on this workspace records the clears ahead of itself.  (With one epoch
+// for all recorded launches every one of them had to clear its words first: three small kernels
+// per call, which made a recorded ring schedule slower than the eager one.)
 int next_epoch(homcomp_workspace *ws, hipStream_t s, uint32_t *epoch)
 {
-    if (stream_is_capturing(s)) {
-        *epoch = kGraphEpoch;
+    unsigned long long capture = 0;
+    if (stream_is_capturing(s, &capture)) {
+        if (capture != ws->capture_id || ws->graph_epoch > kGraphEpochLast) {
+            const int rc = clear_tagged_words(ws, s);
+            if (rc) return rc;
+            ws->capture_id = capture;
+            ws->graph_epoch = kGraphEpochFirst;
+        }
+        *epoch = ws->graph_epoch++;
         return HOMCOMP_OK;
     }
     if (ws->epoch >= kMaxEpoch) {
-        const uint64_t blocks = (uint64_t)ws->max_tiles / 256 + 1;
-        if (!hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)) ||
-            !hip_ok(hc::launch_fill_u64(ws->d_in_blocks[0], blocks, s)) ||
-            !hip_ok(hc::launch_fill_u64(ws->d_in_blocks[1], blocks, s)))
-            return HOMCOMP_ERR_HIP;
+        const int rc = clear_tagged_words(ws, s);
+        if (rc) return rc;
         ws->epoch = 0;
     }
     *epoch = ++ws->epoch;
@@ -130,26 +170,29 @@ int fill_params(homcomp_workspace *ws, size_t n, hipStream_t s, hc::TileParams *
     p->spin_limit = ws->spin_limit;
     p->error = ws->d_error;
     p->total = ws->d_total;
+    // tile offsets handed over for this call (one call only)
+    p->tile_ofs_out = ws->next_out_ofs;
+    p->in_ofs[0] = ws->next_in_ofs[0];
+    p->in_ofs[1] = ws->next_in_ofs[1];
     return next_epoch(ws, s, &p->epoch);
 }
 
 // Offsets pre-pass of the incoming streams (header bytes -> payload offset of every tile): one
-// launch for all of them, under the epoch of the call's tile kernel.
+// launch for all of them, under the epoch of the call's tile kernel.  Streams whose offsets the
+// caller handed over (homcomp_workspace_tile_offsets) need none; the launch is left out when that
+// holds for all of them.
 int in_offsets(homcomp_workspace *ws, int n_streams, hc::TileParams *p, hipStream_t s)
 {
+    const uint64_t *given[2] = {p->in_ofs[0], p->in_ofs[1]};
+    bool all_given = true;
+    for (int c = 0; c < n_streams; ++c) all_given = all_given && given[c] != nullptr;
+    if (all_given) return HOMCOMP_OK;
     hc::InOffsetsArgs a;
     std::memset(&a, 0, sizeof a);
     a.error = ws->d_error;
-    uint32_t epoch = p->epoch;
-    if (stream_is_capturing(s)) {
-        // as for the tile kernel (see chained_launch): a replay finds the words of the replay before
-        epoch = kGraphEpoch;
-        const uint64_t blocks = (uint64_t)p->n_tiles / 256 + 1;
-        for (int c = 0; c < n_streams; ++c)
-            if (!hip_ok(hc::launch_fill_u64(ws->d_in_blocks[c], blocks, s))) return HOMCOMP_ERR_HIP;
-    }
+    const uint32_t epoch = p->epoch;
     for (int c = 0; c < n_streams; ++c) {
-        p->in_ofs[c] = ws->d_in_ofs[c];
+        p->in_ofs[c] = given[c] ? given[c] : ws->d_in_ofs[c];
         a.hdr[c] = p->in[c];
         a.block_words[c] = ws->d_in_blocks[c];
         a.ofs[c] = ws->d_in_ofs[c];
@@ -276,23 +319,15 @@ int spill_release(homcomp_workspace *ws)
     return rc;
 }
 
-// `scan_words` / `n_scan_words`: the scan words of the call, cleared first when the launch is
-// being recorded into a graph.  p.spill == nullptr: the device's spill area is used.
-int chained_launch(int device, uint64_t *scan_words, uint64_t n_scan_words, int op, hc::TileParams p,
-                   uint32_t max_grid, hipStream_t s)
+// p.spill == nullptr: the device's spill area is used.
+int chained_launch(int device, int op, hc::TileParams p, uint32_t max_grid, hipStream_t s)
 {
     const bool capturing = stream_is_capturing(s);
     DeviceState &c = g_dev[device];
     std::lock_guard<std::mutex> lock(c.mu);
     if (!p.spill) p.spill = c.spill;
-    if (capturing) {
-        // A captured launch is replayed with the epoch it was captured with, so the scan words
-        // of the previous replay would read as this call's: the graph clears them first (with
-        // a kernel; memset nodes are avoided in graphs).
-        p.epoch = kGraphEpoch;
-        if (!hip_ok(hc::launch_fill_u64(scan_words, n_scan_words, s))) return HOMCOMP_ERR_HIP;
-        return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
-    }
+    // a stream under capture is left alone: its graph orders the launches it contains
+    if (capturing) return hip_ok(hc::launch_op(op, p, max_grid, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     if (c.any && c.last != s) {
         // The event is recorded only now, on the stream of the previous launch (a call that stays
         // on one stream pays nothing): it covers that launch and whatever followed it there.
@@ -341,6 +376,11 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         p.stage_bytes = 0u;
         return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
+    // Nothing known about the incoming tiles (the size was stated as the buffer's capacity): the
+    // mean tile the operation's last finished call on this workspace produced stands in for them
+    // (a ring step's partial sums resemble those of the step before).
+    const uint64_t seen = *(volatile const uint64_t *)&ws->h_mean_tile[op];   // 0 until a call has finished
+    if (expected_tile_bytes == 0) expected_tile_bytes = seen & 0xffffffffu;
     // stream (+) local operand: the kernel with the bit-plane path where most incoming tiles can
     // take it, else the one without.  The offsets pre-pass counts the tiles of few planes and
     // leaves the count in host-visible memory; it arrives too late for the launch it belongs to,
@@ -369,8 +409,6 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
         } else if (ws->sliced != 0u)
             p.sliced = ws->sliced == 3u ? 2u : 1u;
     }
-    const uint64_t seen = *(volatile const uint64_t *)&ws->h_mean_tile[op];   // 0 until a call has finished
-    if (expected_tile_bytes == 0) expected_tile_bytes = seen & 0xffffffffu;
     int cls = choose_stage_class(op, expected_tile_bytes, ws->out_slots);
     // compress: the budget above holds the mean tile with an eighth to spare.  Tiles that vary
     // (spikes in the data) do not need that: with half of them a little beyond the slots of the
@@ -386,12 +424,14 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
     if (ws->stage_class >= 0) cls = ws->stage_class;
     p.host_total = &ws->h_mean_tile[op];
     p.stage_bytes = kStage[cls][op];
-    return chained_launch(ws->device, ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, op, p, ws->max_grid[op][cls], s);
+    return chained_launch(ws->device, op, p, ws->max_grid[op][cls], s);
 }
 
-// payload bytes per tile of an incoming stream
+// payload bytes per tile of an incoming stream; 0 (unknown) when the stated size is no length but
+// a capacity
 uint64_t tile_bytes_of(const hc::TileParams &p, size_t stream_size)
 {
+    if (stream_size >= homcomp_max_stream_bytes(p.n)) return 0u;
     return stream_size > p.hdr_bytes ? (stream_size - p.hdr_bytes) / p.n_tiles : 1u;
 }
 
@@ -634,6 +674,18 @@ int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value)
     }
 }
 
+size_t homcomp_tile_offsets_count(size_t nbEle) { return padded_len(nbEle) / hc::kHostTileElems; }
+
+int homcomp_workspace_tile_offsets(homcomp_workspace *ws, const uint64_t *d_in_a, const uint64_t *d_in_b, uint64_t *d_out)
+{
+    if (!ws) return HOMCOMP_ERR_INVALID_ARG;
+    if (!aligned16(d_in_a) || !aligned16(d_in_b) || !aligned16(d_out)) return HOMCOMP_ERR_ALIGNMENT;
+    ws->next_in_ofs[0] = d_in_a;
+    ws->next_in_ofs[1] = d_in_b;
+    ws->next_out_ofs = d_out;
+    return HOMCOMP_OK;
+}
+
 int homcomp_workspace_destroy(homcomp_workspace *ws)
 {
     if (!ws) return HOMCOMP_OK;
@@ -650,6 +702,7 @@ int homcomp_compress_f32(homcomp_workspace *ws, const float *d_data, size_t nbEl
                          unsigned char *d_cmp, uint64_t *d_stream_len, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
@@ -670,6 +723,7 @@ int homcomp_compress_plain_f32(homcomp_workspace *ws, const float *d_data, size_
                                unsigned char *d_cmp, uint64_t *d_stream_len, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
@@ -700,6 +754,7 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
                            size_t nbEle, float eb, float *d_out, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
@@ -722,6 +777,7 @@ int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
                         uint64_t *d_stream_len, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (!eb_ok(eb)) return HOMCOMP_ERR_INVALID_ARG;
@@ -746,6 +802,7 @@ int homcomp_hom_sum_i32(homcomp_workspace *ws, const unsigned char *d_cmp_in, si
                         uint64_t *d_stream_len, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
@@ -770,6 +827,7 @@ int homcomp_hom_add(homcomp_workspace *ws, const unsigned char *d_cmp_a, size_t 
                     unsigned char *d_cmp_out, uint64_t *d_stream_len, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    const HandOver hand_over(ws);
     int rc = check_ws(ws, nbEle);
     if (rc) return rc;
     if (nbEle == 0) return empty_stream(ws, d_stream_len, s);
@@ -842,10 +900,7 @@ int homcomp_hom_sum_f32_static(const unsigned char *d_cmp_in, size_t cmp_in_size
         !hip_ok(hc::launch_fill_u64(a.block_words[0], (uint64_t)p.n_tiles / 256 + 1, s)))
         return HOMCOMP_ERR_HIP;
     if (!hip_ok(hc::launch_in_offsets(a, 1, p.n_tiles, p.hdr_bytes, p.epoch, p.spin_limit, s))) return HOMCOMP_ERR_HIP;
-    // (Under capture chained_launch gives the tile kernel the graph's epoch while the pre-pass above
-    // ran under epoch 1.  The two need not agree: the tile kernel never reads the pre-pass's block
-    // words, only the plain offsets it leaves, and both kinds of words were cleared just above.)
-    return chained_launch(device, nullptr, 0, hc::kOpHomSumF32, p, st->grid[cls], s);
+    return chained_launch(device, hc::kOpHomSumF32, p, st->grid[cls], s);
 }
 
 int homcomp_quant_predict_f32(const float *d_data, size_t nbEle, float eb, int32_t *d_delta,

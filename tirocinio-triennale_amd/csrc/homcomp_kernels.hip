@@ -186,8 +186,34 @@ __device__ __forceinline__ void scan_server_steps(const TileParams &p, const Sca
                                                       kBufStatus);
         }
         issue_order();
+        // (what follows comes after the prefixes have gone out: the data waves wait for them)
+        {
+            // The same offsets as plain words for the caller: absolute, header bytes included.
+            // Unconditional like every memory operation of a step (the number of operations between
+            // a request and its look must not depend on the path); without a destination the
+            // window is empty and the stores are dropped.
+            __amdgpu_buffer_rsrc_t ru = words_from(p.tile_ofs_out ? p.tile_ofs_out : c.prefixes, t0);
+            if (!p.tile_ofs_out) ru = buffer_of(c.prefixes, 0);
+            uint64_t at = p.hdr_bytes + base + before + (incl - mine);
+            uint64_t u[PER];
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j) {
+                u[j] = at;
+                at += v[j];
+            }
+            if constexpr (PER == 4) {
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    u32x4{(uint32_t)u[0], (uint32_t)(u[0] >> 32), (uint32_t)u[1], (uint32_t)(u[1] >> 32)}, ru, (int)voff, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    u32x4{(uint32_t)u[2], (uint32_t)(u[2] >> 32), (uint32_t)u[3], (uint32_t)(u[3] >> 32)}, ru, (int)(voff + 16u), 0, 0);
+            } else {
+#pragma unroll
+                for (uint32_t j = 0; j < PER; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b64(u32x2{(uint32_t)u[j], (uint32_t)(u[j] >> 32)}, ru, (int)(voff + 8u * j), 0, 0);
+            }
+            issue_order();
+        }
         base += step_total;
-        // (after the prefixes have gone out: the data waves wait for them)
         if (p.probe_bytes != 0u) {
 #pragma unroll
             for (uint32_t j = 0; j < PER; ++j) over += v[j] > p.probe_bytes ? 1u : 0u;

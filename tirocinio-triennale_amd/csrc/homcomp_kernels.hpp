@@ -38,6 +38,8 @@ struct TileParams {
     uint32_t *error;            // sticky error flags (bit 0: scan wait gave up)
     uint64_t *total;            // receives the stream length
     uint64_t *user_total;       // optional second destination for the stream length
+    uint64_t *tile_ofs_out;     // optional: receives, per tile of the outgoing stream, the absolute byte offset of the tile's
+                                // payload (what in_ofs holds for an incoming stream), n_tiles plain words
     uint8_t *spill;             // out_slots slots of kSpillSlotBytes per data wave, for tiles that outgrow their LDS slot
     uint32_t out_slots;         // rounds a packed tile waits in LDS for its stream offset: 2 to 4
     uint32_t sliced;            // the sums' bit-plane paths.  0: no tile takes one (stream (+) local operand then runs the

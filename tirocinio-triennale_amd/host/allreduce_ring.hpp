@@ -23,7 +23,11 @@
 //     the array (count far below its multiple of 32768) the reference's block count goes
 //     negative; here that block is empty and the blocks before it carry the padding;
 //   * buffers and the workspace can be kept between calls (RingBuffers), which is what the
-//     reference's _opt variant does by hand (:745-760).
+//     reference's _opt variant does by hand (:745-760);
+//   * a message is the stream preceded by its tile offsets (8 bytes per 4096 elements of the
+//     block, homcomp_workspace_tile_offsets): the call that produced the stream leaves them in
+//     front of it, and the receiving rank's call takes them from there instead of scanning the
+//     header bytes first (a launch of its own, a third of a ring step's call).
 // Returns 0, or the first non-zero status (HOMCOMP_ERR_* or the communicator's).
 #pragma once
 
@@ -111,7 +115,8 @@ public:
     {
         if (padded <= cap_padded_ && max_block <= cap_block_ && (!int_deltas || d_quant)) return HOMCOMP_OK;
         release();
-        stream_cap = homcomp_max_stream_bytes(max_block);
+        // a message: the tile offsets of the block's stream, then the stream
+        stream_cap = homcomp_tile_offsets_count(max_block) * sizeof(uint64_t) + homcomp_max_stream_bytes(max_block);
         bool ok = hipMalloc((void **)&d_rtmpbuf, (padded ? padded : 1) * sizeof(float)) == hipSuccess;
         ok = ok && hipMalloc((void **)&d_cmpReduceBytes, stream_cap + HOMCOMP_STREAM_SLACK) == hipSuccess;
         ok = ok && hipMalloc((void **)&d_inbuf[0], stream_cap + HOMCOMP_STREAM_SLACK) == hipSuccess;
@@ -136,7 +141,7 @@ public:
     unsigned char *d_inbuf[2] = {nullptr, nullptr};
     int *d_quant = nullptr;
     homcomp_workspace *ws = nullptr;
-    size_t stream_cap = 0;
+    size_t stream_cap = 0;   // capacity of a message buffer
 
 private:
     void release()
@@ -178,26 +183,57 @@ struct RingCall {
         rc = launch();
         return rc != HOMCOMP_OK ? rc : homcomp_last_size(buf.ws, len, stream);
     }
-    // GSZ_compress_deviceptr_outlier
-    int compress(const float *d_block, size_t n, unsigned char *d_out, size_t *len) const
+    // A message buffer holds the tile offsets of the block's stream, then the stream.
+    static size_t ofs_bytes(size_t n) { return homcomp_tile_offsets_count(n) * sizeof(uint64_t); }
+    static uint64_t *ofs_of(unsigned char *d_msg) { return reinterpret_cast<uint64_t *>(d_msg); }
+    static const uint64_t *ofs_of(const unsigned char *d_msg) { return reinterpret_cast<const uint64_t *>(d_msg); }
+    // A stream-producing call into the message buffer d_out, reading the message d_in (or none);
+    // *msg_len = offsets + stream.  (The hand-over of the offsets is one call's: it is made again
+    // when a timed-out call is repeated.)
+    template <typename Launch>
+    int produce(Launch launch, size_t n, const unsigned char *d_in, unsigned char *d_out, size_t *msg_len) const
     {
-        return sized([&] { return homcomp_compress_f32(buf.ws, d_block, n, eb, d_out, nullptr, stream); }, len);
+        size_t len = 0;
+        const int rc = sized(
+            [&] {
+                const int ro = homcomp_workspace_tile_offsets(buf.ws, n && d_in ? ofs_of(d_in) : nullptr, nullptr,
+                                                              n ? ofs_of(d_out) : nullptr);
+                return ro != HOMCOMP_OK ? ro : launch(d_out + ofs_bytes(n));
+            },
+            &len);
+        *msg_len = ofs_bytes(n) + len;
+        return rc;
     }
-    // homomorphic_sum_F, or kernel_quant_prediction + homomorphic_sum (:61-72)
-    int hom_sum(const unsigned char *d_in, size_t in_len, const float *d_block, size_t n, unsigned char *d_out,
-                size_t *len) const
+    // GSZ_compress_deviceptr_outlier
+    int compress(const float *d_block, size_t n, unsigned char *d_out, size_t *msg_len) const
     {
+        return produce([&](unsigned char *d_cmp) { return homcomp_compress_f32(buf.ws, d_block, n, eb, d_cmp, nullptr, stream); }, n,
+                       nullptr, d_out, msg_len);
+    }
+    // homomorphic_sum_F, or kernel_quant_prediction + homomorphic_sum (:61-72), on a received message
+    int hom_sum(const unsigned char *d_in, size_t in_msg_len, const float *d_block, size_t n, unsigned char *d_out,
+                size_t *msg_len) const
+    {
+        if (in_msg_len < ofs_bytes(n)) return HOMCOMP_ERR_INVALID_ARG;
+        const unsigned char *d_cmp_in = d_in + ofs_bytes(n);
+        const size_t in_len = in_msg_len - ofs_bytes(n);
         if (int_deltas) {
             const int rc = homcomp_quant_predict_f32(d_block, n, eb, buf.d_quant, stream);
             if (rc != HOMCOMP_OK) return rc;
-            return sized([&] { return homcomp_hom_sum_i32(buf.ws, d_in, in_len, buf.d_quant, n, d_out, nullptr, stream); },
-                         len);
         }
-        return sized([&] { return homcomp_hom_sum_f32(buf.ws, d_in, in_len, d_block, n, eb, d_out, nullptr, stream); }, len);
+        return produce(
+            [&](unsigned char *d_cmp) {
+                return int_deltas ? homcomp_hom_sum_i32(buf.ws, d_cmp_in, in_len, buf.d_quant, n, d_cmp, nullptr, stream)
+                                  : homcomp_hom_sum_f32(buf.ws, d_cmp_in, in_len, d_block, n, eb, d_cmp, nullptr, stream);
+            },
+            n, d_in, d_out, msg_len);
     }
-    int decompress(const unsigned char *d_in, size_t in_len, float *d_block, size_t n) const
+    int decompress(const unsigned char *d_in, size_t in_msg_len, float *d_block, size_t n) const
     {
-        const int rc = homcomp_decompress_f32(buf.ws, d_in, in_len, n, eb, d_block, stream);
+        if (in_msg_len < ofs_bytes(n)) return HOMCOMP_ERR_INVALID_ARG;
+        int rc = homcomp_workspace_tile_offsets(buf.ws, n ? ofs_of(d_in) : nullptr, nullptr, nullptr);
+        if (rc == HOMCOMP_OK)
+            rc = homcomp_decompress_f32(buf.ws, d_in + ofs_bytes(n), in_msg_len - ofs_bytes(n), n, eb, d_block, stream);
         if (rc != HOMCOMP_OK) return rc;
         return hipStreamSynchronize(stream) == hipSuccess ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
     }
