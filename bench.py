@@ -100,7 +100,7 @@ def sweep(torch, pkg, gen) -> int:
         n = 1 << log2n
         ws = pkg.Workspace(n)
         cap = pkg.max_stream_bytes(n)
-        bufs = [torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(3)]
+        bufs = [torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda") for _ in range(3)]
         dec = torch.empty(n, dtype=torch.float32, device="cuda")
         mm = torch.empty(4, dtype=torch.float32, device="cuda")
         for kind in ("smooth", "gradient_like", "uniform"):
@@ -162,9 +162,12 @@ def error_measures(torch, x, y, dec, eb, chunk=1 << 24):
             "correlation": round(cov / math.sqrt(var_o * var_d), 9) if var_o > 0 and var_d > 0 else None}
 
 
-def op_entry(n, ms, alg_bytes):
-    return {"ms": round(ms, 4), "GBps_input": round(4 * n / ms / 1e6, 1),
-            "frac_hbm": round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)}
+def op_entry(n, ms, alg_bytes, ws=None):
+    e = {"ms": round(ms, 4), "GBps_input": round(4 * n / ms / 1e6, 1),
+         "frac_hbm": round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)}
+    if ws is not None:
+        e.update(ws.last_launch())   # kernel kind and LDS budget the timed calls ran with
+    return e
 
 
 def other_configs(torch, pkg, gen, orc):
@@ -199,7 +202,7 @@ def other_configs(torch, pkg, gen, orc):
     ws.value_range(x, mm)
     r = mm.cpu().numpy()
     cap = pkg.max_stream_bytes(n)
-    ca = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    ca = torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda")
     dec = torch.empty(n, dtype=torch.float32, device="cuda")
     xh = x.cpu().numpy() if orc is not None else None
     for rel in (1e-4, 1e-3):
@@ -207,7 +210,7 @@ def other_configs(torch, pkg, gen, orc):
         ws.compress(x, eb, ca)
         la = ws.last_size()
         e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3),
-             "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10, warm=2), 4 * n + la),
+             "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10, warm=2), 4 * n + la, ws),
              "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(ca, la, n, eb, dec), 10, warm=2), la + 4 * n)}
         if orc is not None:
             want = orc.compress(xh, np.float32(eb))
@@ -229,7 +232,7 @@ def other_configs(torch, pkg, gen, orc):
     y = gen.gradient_like_torch(n, seed=2)
     ws = pkg.Workspace(n)
     cap = pkg.max_stream_bytes(n)
-    ca, cb, cs = (torch.empty(cap, dtype=torch.uint8, device="cuda") for _ in range(3))
+    ca, cb, cs = (torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda") for _ in range(3))
     dec = torch.empty(n, dtype=torch.float32, device="cuda")
     ws.compress(x, eb, ca)
     la = ws.last_size()
@@ -237,12 +240,15 @@ def other_configs(torch, pkg, gen, orc):
     lb = ws.last_size()
     ws.hom_sum_f32(ca, la, y, eb, cs)
     ls = ws.last_size()
+    # The workspace picks kernel kind and LDS budget from what its earlier calls saw, so a timing
+    # depends on the calls before it; every operation is timed after the same warm sequence (ten
+    # untimed calls of itself, by which the choice has settled), and the choice is reported.
     e = {"elements": n, "eb_abs": eb, "compression_ratio": round(4 * n / la, 3), "compression_ratio_sum": round(4 * n / ls, 3),
-         "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 5, warm=2), 4 * n + la),
-         "hom_sum_f32": op_entry(n, time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), 5, warm=2), la + 4 * n + ls),
-         "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), 5, warm=2), ls + 4 * n)}
+         "compress": op_entry(n, time_op(torch, lambda: ws.compress(x, eb, ca), 10, warm=10), 4 * n + la, ws),
+         "hom_sum_f32": op_entry(n, time_op(torch, lambda: ws.hom_sum_f32(ca, la, y, eb, cs), 10, warm=10), la + 4 * n + ls, ws),
+         "decompress": op_entry(n, time_op(torch, lambda: ws.decompress(cs, ls, n, eb, dec), 10, warm=10), ls + 4 * n)}
     ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8))   # dec doubles as the output buffer: 4N >= L here
-    e["hom_add"] = op_entry(n, time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8)), 5, warm=2), la + lb + ls)
+    e["hom_add"] = op_entry(n, time_op(torch, lambda: ws.hom_add(ca, la, cb, lb, n, dec.view(torch.uint8)), 10, warm=10), la + lb + ls, ws)
     ok = ws.last_size() == ls and bool(torch.equal(dec.view(torch.uint8)[:ls], cs[:ls]))
     e["hom_add_equals_hom_sum_f32"] = ok
     if orc is not None:
@@ -407,9 +413,9 @@ def main() -> int:
     eb = float(args.abs) if args.abs is not None else pkg.rel_to_abs(args.rel, vmin, vmax)
 
     cap = pkg.max_stream_bytes(n)
-    cmp_a = torch.empty(cap, dtype=torch.uint8, device="cuda")
-    cmp_b = torch.empty(cap, dtype=torch.uint8, device="cuda")
-    cmp_s = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    cmp_a = torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda")
+    cmp_b = torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda")
+    cmp_s = torch.empty(cap + pkg.STREAM_SLACK, dtype=torch.uint8, device="cuda")
     dec = torch.empty(n, dtype=torch.float32, device="cuda")
 
     ws.compress(x, eb, cmp_a)
@@ -437,22 +443,24 @@ def main() -> int:
     it = max(5, args.steps)
     ops = {}
 
-    def add(name, fn, alg_bytes):
-        ms = time_op(torch, fn, it)
+    def add(name, fn, alg_bytes, producing=True):
+        ms = time_op(torch, fn, it, warm=3)
         ops[name] = {"ms": round(ms, 4), "GBps_input": round(4 * n / ms / 1e6, 1),
                      "alg_bytes": int(alg_bytes),
                      "achieved_GBps": round(alg_bytes / ms / 1e6, 1),
                      "frac_hbm": round(alg_bytes / (ms * 1e-3) / HBM_PEAK, 4)}
+        if producing:
+            ops[name].update(ws.last_launch())   # kernel kind and LDS budget the timed calls ran with
 
     add("compress", lambda: ws.compress(x, eb, cmp_a), 4 * n + la)
     add("hom_sum_f32", lambda: ws.hom_sum_f32(cmp_a, la, y, eb, cmp_s), la + 4 * n + ls)
-    add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n)
+    add("decompress", lambda: ws.decompress(cmp_s, ls, n, eb, dec), ls + 4 * n, producing=False)
     add("hom_add", lambda: ws.hom_add(cmp_a, la, cmp_b, lb, n, cmp_s), la + lb + ls)
     # the integer-delta variant of the sum with its Lorenzo pre-pass, and the min/max scan behind REL bounds
     dlt = torch.empty(n, dtype=torch.int32, device="cuda")
-    add("quant_predict", lambda: pkg.quant_predict(y, eb, dlt), 8 * n)
+    add("quant_predict", lambda: pkg.quant_predict(y, eb, dlt), 8 * n, producing=False)
     add("hom_sum_i32", lambda: ws.hom_sum_i32(cmp_a, la, dlt, cmp_b), la + 4 * n + ls)
-    add("value_range", lambda: ws.value_range(x, mm[0:2]), 4 * n)
+    add("value_range", lambda: ws.value_range(x, mm[0:2]), 4 * n, producing=False)
     del dlt
     ws.compress(y, eb, cmp_b)   # cmp_b holds compress(y) again
     torch.cuda.synchronize()

@@ -88,10 +88,27 @@ int homcomp_workspace_destroy(homcomp_workspace *ws);
  *       where other kernels hold compute units for longer than the bounded waits (tens of
  *       milliseconds) a full grid ends in HOMCOMP_ERR_SCAN_TIMEOUT, a smaller one fits beside them.
  *   HOMCOMP_OPT_SPIN_LIMIT    unsuccessful re-reads of a scan word before a wave gives up, 0..2^30
- *       (default 65536, or HOMCOMP_SPIN_LIMIT at creation). */
+ *       (default 65536, or HOMCOMP_SPIN_LIMIT at creation).
+ *   HOMCOMP_OPT_LDS_BUDGET    LDS stage per data wave of the stream-producing kernels: -1 (default) chosen
+ *       per call from the size of the tiles the workspace has seen (so the time of a call can depend
+ *       on the calls before it, never its bytes), 0 / 1 / 2 = always the small / medium / large one
+ *       (4 / 3 / 2 workgroups per compute unit; HOMCOMP_STAGE=small|medium|large at creation).
+ *   HOMCOMP_OPT_PLANE_PATHS   which kernel kind the homomorphic sums run: 1 (default) chosen per call
+ *       from the plane counts of the streams the workspace has seen, 0 = the general path only, 2 =
+ *       always the kernels with the path for blocks of few planes, 3 = stream (+) stream always the
+ *       kernel for wide blocks (HOMCOMP_SLICED=0..3 at creation).  Every kind gives the same bytes.
+ * Fixing the last two makes timings independent of the workspace's history. */
 #define HOMCOMP_OPT_GRID_PERCENT 1
 #define HOMCOMP_OPT_SPIN_LIMIT 2
+#define HOMCOMP_OPT_LDS_BUDGET 3
+#define HOMCOMP_OPT_PLANE_PATHS 4
 int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value);
+/* What the last stream-producing call on ws was launched with: the kernel kind and the LDS budget
+ * (0 small, 1 medium, 2 large); -1 before the first such call.  Either pointer may be NULL. */
+#define HOMCOMP_KERNEL_GENERAL 0
+#define HOMCOMP_KERNEL_FEW_PLANES 1
+#define HOMCOMP_KERNEL_WIDE_PLANES 2
+int homcomp_workspace_last_launch(const homcomp_workspace *ws, int *kernel_kind, int *lds_budget);
 
 /* Tile offsets: a side array that spares the call that reads a stream its pass over the header
  * bytes.  The payload position of a block follows from the header bytes of all blocks before it

@@ -19,7 +19,7 @@ EXPORTS = (
     "homcomp_status_string", "homcomp_last_hip_error", "homcomp_header_bytes",
     "homcomp_max_stream_bytes", "homcomp_ref_cmpsize", "homcomp_workspace_create",
     "homcomp_workspace_destroy", "homcomp_workspace_set_option", "homcomp_tile_offsets_count",
-    "homcomp_workspace_tile_offsets", "homcomp_compress_f32", "homcomp_decompress_f32",
+    "homcomp_workspace_tile_offsets", "homcomp_workspace_last_launch", "homcomp_compress_f32", "homcomp_decompress_f32",
     "homcomp_compress_plain_f32", "homcomp_decompress_plain_f32",
     "homcomp_hom_sum_f32", "homcomp_hom_sum_i32", "homcomp_hom_add", "homcomp_hom_sum_f32_static",
     "homcomp_quant_predict_f32", "homcomp_range_f32", "homcomp_rel_to_abs", "homcomp_last_size",
@@ -28,6 +28,10 @@ EXPORTS = (
 
 OPT_GRID_PERCENT = 1
 OPT_SPIN_LIMIT = 2
+OPT_LDS_BUDGET = 3      # -1 automatic, 0 small, 1 medium, 2 large
+OPT_PLANE_PATHS = 4     # 1 automatic, 0 general path only, 2 few-plane kernels, 3 wide-block kernel for stream (+) stream
+KERNEL_KINDS = {-1: None, 0: "general", 1: "few_planes", 2: "wide_planes"}
+LDS_BUDGETS = {-1: None, 0: "small", 1: "medium", 2: "large"}
 ERR_SCAN_TIMEOUT = -6
 
 
@@ -69,6 +73,7 @@ def lib() -> C.CDLL:
         L.homcomp_tile_offsets_count.argtypes = [sz]
         L.homcomp_tile_offsets_count.restype = sz
         L.homcomp_workspace_tile_offsets.argtypes = [vp, vp, vp, vp]
+        L.homcomp_workspace_last_launch.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.homcomp_compress_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
         L.homcomp_decompress_f32.argtypes = [vp, vp, sz, sz, C.c_float, vp, vp]
         L.homcomp_compress_plain_f32.argtypes = [vp, vp, sz, C.c_float, vp, u64p, vp]
@@ -143,6 +148,12 @@ class Workspace:
 
     def set_option(self, option: int, value: int) -> None:
         _check(lib().homcomp_workspace_set_option(self._h, int(option), int(value)), "workspace_set_option")
+
+    def last_launch(self) -> dict:
+        """Kernel kind and LDS budget of the last stream-producing call on this workspace."""
+        kind, budget = C.c_int(), C.c_int()
+        _check(lib().homcomp_workspace_last_launch(self._h, C.byref(kind), C.byref(budget)), "workspace_last_launch")
+        return {"kernel": KERNEL_KINDS[kind.value], "lds_budget": LDS_BUDGETS[budget.value]}
 
     def tile_offsets(self, in_a=None, in_b=None, out=None) -> None:
         """Tile offsets for the next call on this workspace (homcomp_workspace_tile_offsets): int64 device

@@ -103,7 +103,9 @@ def check_spills(table: dict[str, dict[str, int]]) -> list[str]:
     return bad
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, enforce: bool = True) -> str:
+    """enforce=False (``--allow-spills`` on the command line): report violations of the no-spill
+    rule instead of failing, for experiments."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, *FLAGS, *REMARKS, "-o", LIB, *SOURCES]
     if verbose:
@@ -117,7 +119,9 @@ def build(verbose: bool = False) -> str:
     with open(RESOURCES, "w") as f:
         f.write(resource_table(table))
     bad = check_spills(table)
-    if bad:
+    if bad and not enforce:
+        print("NOT ENFORCED: " + "; ".join(bad), file=sys.stderr)
+    elif bad:
         os.remove(LIB)
         raise RuntimeError("tile kernels must not spill vector registers:\n  " + "\n  ".join(bad))
     if verbose:
@@ -131,4 +135,4 @@ def build(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, enforce="--allow-spills" not in sys.argv[1:]))

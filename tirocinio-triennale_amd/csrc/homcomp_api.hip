@@ -80,6 +80,7 @@ struct homcomp_workspace {
                               // kernels with the path for few planes whatever the streams look like; 3: stream (+) stream
                               // runs the kernel for wide blocks whatever the streams look like
     int stage_class;          // -1: chosen per call; 0 / 1 / 2: HOMCOMP_STAGE=small / medium / large forces one LDS budget
+    int last_kind, last_budget;   // what the last stream-producing call was launched with (homcomp_workspace_last_launch)
 };
 
 namespace {
@@ -424,6 +425,9 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
     if (ws->stage_class >= 0) cls = ws->stage_class;
     p.host_total = &ws->h_mean_tile[op];
     p.stage_bytes = kStage[cls][op];
+    ws->last_budget = cls;
+    ws->last_kind = op == hc::kOpCompress ? HOMCOMP_KERNEL_GENERAL
+                                          : (p.sliced == 2u ? HOMCOMP_KERNEL_WIDE_PLANES : (p.sliced ? HOMCOMP_KERNEL_FEW_PLANES : HOMCOMP_KERNEL_GENERAL));
     return chained_launch(ws->device, op, p, ws->max_grid[op][cls], s);
 }
 
@@ -606,6 +610,7 @@ int homcomp_workspace_create(homcomp_workspace **out, size_t max_nbEle)
         if (waves > ws->max_tiles) waves = ws->max_tiles;
         ok = spill_acquire(ws, waves * ws->out_slots * hc::kSpillSlotBytes) == HOMCOMP_OK;
     }
+    ws->last_kind = ws->last_budget = -1;
     ws->stage_class = -1;
     if (const char *e = std::getenv("HOMCOMP_STAGE")) {
         if (std::strcmp(e, "small") == 0) ws->stage_class = 0;
@@ -669,9 +674,25 @@ int homcomp_workspace_set_option(homcomp_workspace *ws, int option, long value)
         if (value < 0 || value > (1l << 30)) return HOMCOMP_ERR_INVALID_ARG;
         ws->spin_limit = (uint32_t)value;
         return HOMCOMP_OK;
+    case HOMCOMP_OPT_LDS_BUDGET:
+        if (value < -1 || value >= kStageClasses) return HOMCOMP_ERR_INVALID_ARG;
+        ws->stage_class = (int)value;
+        return HOMCOMP_OK;
+    case HOMCOMP_OPT_PLANE_PATHS:
+        if (value < 0 || value > 3) return HOMCOMP_ERR_INVALID_ARG;
+        ws->sliced = (uint32_t)value;
+        return HOMCOMP_OK;
     default:
         return HOMCOMP_ERR_INVALID_ARG;
     }
+}
+
+int homcomp_workspace_last_launch(const homcomp_workspace *ws, int *kernel_kind, int *lds_budget)
+{
+    if (!ws) return HOMCOMP_ERR_INVALID_ARG;
+    if (kernel_kind) *kernel_kind = ws->last_kind;
+    if (lds_budget) *lds_budget = ws->last_budget;
+    return HOMCOMP_OK;
 }
 
 size_t homcomp_tile_offsets_count(size_t nbEle) { return padded_len(nbEle) / hc::kHostTileElems; }
