@@ -27,7 +27,7 @@ def test_fixed_budget_and_kernel_kind(pkg, cuda, orc, gen):
             assert np.array_equal(got, sa), f"compress, budget {name}: {first_diff(got, sa)}"
             launched = g.ws.last_launch()
             assert launched["kernel"] == "general" and (name is None or launched["lds_budget"] == name)
-            for paths, kinds in ((0, ("general", "general")), (2, ("few_planes", "few_planes")), (3, ("few_planes", "wide_planes")),
+            for paths, kinds in ((0, ("general", "general")), (2, ("few_planes", "few_planes")), (3, (None, "wide_planes")),
                                  (1, (None, None))):
                 g.ws.set_option(pkg.OPT_PLANE_PATHS, paths)
                 got = g.hom_sum_f32(sa, b, eb)

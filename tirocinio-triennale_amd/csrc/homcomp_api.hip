@@ -426,8 +426,10 @@ int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expec
     p.host_total = &ws->h_mean_tile[op];
     p.stage_bytes = kStage[cls][op];
     ws->last_budget = cls;
-    ws->last_kind = op == hc::kOpCompress ? HOMCOMP_KERNEL_GENERAL
-                                          : (p.sliced == 2u ? HOMCOMP_KERNEL_WIDE_PLANES : (p.sliced ? HOMCOMP_KERNEL_FEW_PLANES : HOMCOMP_KERNEL_GENERAL));
+    if (op == hc::kOpCompress || p.sliced == 0u)
+        ws->last_kind = HOMCOMP_KERNEL_GENERAL;
+    else
+        ws->last_kind = op == hc::kOpHomAdd && p.sliced == 2u ? HOMCOMP_KERNEL_WIDE_PLANES : HOMCOMP_KERNEL_FEW_PLANES;
     return chained_launch(ws->device, op, p, ws->max_grid[op][cls], s);
 }
 
