@@ -368,14 +368,34 @@ int choose_stage_class(int op, uint64_t expected_tile_bytes, uint32_t out_slots)
     return holds < 0 || holds == kStageClasses - 1 ? 0 : holds;
 }
 
-// expected_tile_bytes: payload bytes per tile the call is expected to produce, 0 if unknown
+// Grid of the decoder.  The decoder is bound by its stores (2 KiB per wave and sub-step, each
+// wave waiting for its own), and with every wave slot of the device taken they queue up behind
+// each other: measured on MI355X at 64M and 256M elements over three data families and five
+// bounds, streams of up to about 2.5 KB per tile (compressed 6.5 times and better, payload in most
+// blocks) decode 9-13 % faster on 44 % of the resident grid (five waves per compute unit in two,
+// 199 against 229 us for 1 GiB), streams of 2.5-4.2 KB per tile 8 % faster on half of it; longer
+// tiles need every wave for their loads, and streams of almost empty tiles (below 300 bytes) do
+// not care.  Calls of less than two rounds of the full grid keep it.  A heuristic for speed only:
+// any grid gives the same values.
+uint32_t decoder_grid(uint32_t full, uint32_t n_tiles, uint64_t tile_bytes)
+{
+    if ((uint64_t)n_tiles < 2ull * 4u * full) return full;
+    uint32_t percent = 100;
+    if (tile_bytes >= 300u && tile_bytes <= 2560u) percent = 44;
+    else if (tile_bytes > 2560u && tile_bytes <= 4200u) percent = 50;
+    const uint32_t g = (uint32_t)((uint64_t)full * percent / 100u);
+    return g ? g : 1u;
+}
+
+// expected_tile_bytes: payload bytes per tile the call is expected to produce (the decoder: to read), 0 if unknown
 int run_tile_op(homcomp_workspace *ws, int op, hc::TileParams &p, uint64_t expected_tile_bytes, hipStream_t s)
 {
     p.out_slots = ws->out_slots;
     p.sliced = ws->sliced == 3u ? 1u : ws->sliced;
     if (op == hc::kOpDecompress) {
         p.stage_bytes = 0u;
-        return hip_ok(hc::launch_op(op, p, ws->max_grid[op][0], s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
+        return hip_ok(hc::launch_op(op, p, decoder_grid(ws->max_grid[op][0], p.n_tiles, expected_tile_bytes), s)) ? HOMCOMP_OK
+                                                                                                                    : HOMCOMP_ERR_HIP;
     }
     // Nothing known about the incoming tiles (the size was stated as the buffer's capacity): the
     // mean tile the operation's last finished call on this workspace produced stands in for them
@@ -792,7 +812,7 @@ int homcomp_decompress_f32(homcomp_workspace *ws, const unsigned char *d_cmp, si
     p.eb = eb;
     p.recip = 0.5f / eb;
     if ((rc = in_offsets(ws, 1, &p, s))) return rc;
-    return run_tile_op(ws, hc::kOpDecompress, p, 0, s);
+    return run_tile_op(ws, hc::kOpDecompress, p, tile_bytes_of(p, cmp_size), s);
 }
 
 int homcomp_hom_sum_f32(homcomp_workspace *ws, const unsigned char *d_cmp_in, size_t cmp_in_size,
