@@ -141,3 +141,24 @@ def test_plain_codec_at_size(pkg, cuda, orc, gen, kind, log2n, rel):
         ws.close()
         del x
         torch.cuda.empty_cache()
+
+
+def test_plain_decoder_reads_no_further_than_the_stream(gpu, orc, gen):
+    """The plain decoder is told no size: it reads what the header bytes describe, in aligned 16-byte
+    pieces.  A buffer that ends at the 16-byte boundary behind the stream's last byte is enough,
+    and what lies in the rest of that last piece does not matter."""
+    torch = gpu.torch
+    n = (1 << 17) + 4099
+    x = gen.uniform_np(n, 9)
+    eb = np.float32(1e-4)
+    s = orc.compress_plain(x, eb)
+    want = orc.decompress_plain(s, n, eb)
+    for fill in (0x00, 0xFF, 0x5A):
+        for shift in (0, 5):            # the stream's start at two alignments inside the allocation
+            room = (s.size + shift + 15) // 16 * 16
+            buf = torch.full((room,), fill, dtype=torch.uint8, device="cuda")
+            buf[shift:shift + s.size] = torch.from_numpy(s).cuda()
+            out = torch.full((n,), 7.0, dtype=torch.float32, device="cuda")
+            gpu.ws.decompress_plain(buf[shift:], n, float(eb), out)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), (fill, shift)

@@ -121,14 +121,13 @@ bool stream_is_capturing(hipStream_t s, unsigned long long *id = nullptr)
     return cap != hipStreamCaptureStatusNone;
 }
 
+// One fill over everything between the first scan word and the last pre-pass word (the tile offsets
+// of the incoming streams lie between them; they are rewritten by every call that uses them).
 int clear_tagged_words(homcomp_workspace *ws, hipStream_t s)
 {
     const uint64_t blocks = (uint64_t)ws->max_tiles / 256 + 1;
-    return hip_ok(hc::launch_fill_u64(ws->d_tile_totals, (uint64_t)ws->max_tiles * 2, s)) &&
-                   hip_ok(hc::launch_fill_u64(ws->d_in_blocks[0], blocks, s)) &&
-                   hip_ok(hc::launch_fill_u64(ws->d_in_blocks[1], blocks, s))
-               ? HOMCOMP_OK
-               : HOMCOMP_ERR_HIP;
+    const uint64_t words = (uint64_t)((ws->d_in_blocks[1] + blocks) - ws->d_tile_totals);
+    return hip_ok(hc::launch_fill_u64(ws->d_tile_totals, words, s)) ? HOMCOMP_OK : HOMCOMP_ERR_HIP;
 }
 
 // Fresh epoch for one launch; clears the scan words (the two arrays are adjacent) and the block
