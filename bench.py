@@ -133,6 +133,40 @@ def sweep(torch, pkg, gen) -> int:
     return 0
 
 
+def sweep_decoder_grid(torch, pkg, gen) -> int:
+    """Decompress time against the share of the resident grid the decoder is launched with
+    (HOMCOMP_OPT_GRID_PERCENT on top of the library's own choice, which the first column shows):
+    2^24 .. 2^28 elements x three kinds x five REL bounds, one JSON line per point."""
+    for log2n in (28, 26, 24):
+        n = 1 << log2n
+        ws = pkg.Workspace(n)
+        cap = pkg.max_stream_bytes(n) + pkg.STREAM_SLACK
+        ca = torch.empty(cap, dtype=torch.uint8, device="cuda")
+        dec = torch.empty(n, dtype=torch.float32, device="cuda")
+        mm = torch.empty(2, dtype=torch.float32, device="cuda")
+        for kind in ("smooth", "gradient_like", "uniform"):
+            x = gen.GENERATORS_TORCH[kind](n, seed=1)
+            ws.value_range(x, mm)
+            r = mm.cpu().numpy()
+            for rel in (1e-2, 1e-3, 1e-4, 1e-5, 1e-6):
+                eb = pkg.rel_to_abs(rel, float(r[0]), float(r[1]))
+                ws.set_option(pkg.OPT_GRID_PERCENT, 100)
+                ws.compress(x, eb, ca)
+                la = ws.last_size()
+                pt = {"log2n": log2n, "kind": kind, "rel": rel, "CR": round(4 * n / la, 2),
+                      "payload_bytes_per_tile": (la - pkg.header_bytes(n)) // (n // 4096)}
+                # the library's choice (the size is stated), then the whole resident grid and shares of it (the size stated
+                # as the capacity switches the library's choice off)
+                pt["library_us"] = round(min(time_op(torch, lambda: ws.decompress(ca, la, n, eb, dec), 20, warm=5) for _ in range(2)) * 1e3, 1)
+                for pct in (100, 67, 50, 44, 33):
+                    ws.set_option(pkg.OPT_GRID_PERCENT, pct)
+                    t = min(time_op(torch, lambda: ws.decompress(ca, cap, n, eb, dec), 20, warm=5) for _ in range(2))
+                    pt[f"us_at_{pct}"] = round(t * 1e3, 1)
+                print(json.dumps(pt), flush=True)
+        ws.close()
+    return 0
+
+
 def error_measures(torch, x, y, dec, eb, chunk=1 << 24):
     """Maximum absolute error, PSNR, NRMSE and correlation of dec against the exact x + y (float64),
     accumulated chunk by chunk on the GPU; two operands, so the bound is 2 * eb."""
@@ -383,6 +417,8 @@ def main() -> int:
                     help="only the headline workload (profiling runs); default: the other named configurations follow it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1:1 copy of an operand (reference point for HBM counters)")
+    ap.add_argument("--sweep-decoder-grid", action="store_true",
+                    help="instead of the benchmark line: decompress time against the decoder's share of the resident grid")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark line: sizes x data families x REL bounds, one JSON line per point")
     args = ap.parse_args()
@@ -399,6 +435,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     if args.sweep:
         return sweep(torch, pkg, gen)
+    if args.sweep_decoder_grid:
+        return sweep_decoder_grid(torch, pkg, gen)
     n = 1 << args.log2n
     x = gen.GENERATORS_TORCH[args.kind](n, seed=1)
     y = gen.GENERATORS_TORCH[args.kind](n, seed=2)
