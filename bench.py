@@ -593,4 +593,16 @@ def main() -> int:
 
 
 if __name__ == "__main__":
-    sys.exit(main())
+    try:
+        sys.exit(main())
+    except SystemExit:
+        raise
+    except BaseException:
+        # An exception leaves device tensors alive in its traceback; released during interpreter
+        # shutdown they have ended the process in an abort on this stack, which from outside looks
+        # like a GPU fault.  Report and leave without the shutdown.
+        import traceback
+        traceback.print_exc()
+        sys.stdout.flush()
+        sys.stderr.flush()
+        os._exit(1)

@@ -77,7 +77,12 @@ def check_point(pt, full_oracle=True, properties=True):
     pt.same(ca, la, want_a, "compress")
     want_s = orc.hom_sum_f32(want_a, yh, eb)
     pt.same(cs, ls, want_s, "hom_sum_f32")
-    # the Lorenzo pre-pass and the sum with its int32 deltas (HomComp/src/homcomp.cu:1553-1602, 1604-2921)
+    if full_oracle:
+        want_b = orc.compress(yh, eb)
+        pt.same(cb, lb, want_b, "compress (second operand)")
+        pt.same(cs2, ls2, orc.hom_add(want_a, want_b, n), "hom_add")
+    # the Lorenzo pre-pass and the sum with its int32 deltas (HomComp/src/homcomp.cu:1553-1602, 1604-2921);
+    # cs2 held hom_add's stream until here
     dlt = torch.full((n,), 12345, dtype=torch.int32, device="cuda")
     pt.pkg.quant_predict(pt.y, float(eb), dlt)
     ws.hom_sum_i32(ca, la, dlt, cs2)
@@ -86,10 +91,6 @@ def check_point(pt, full_oracle=True, properties=True):
     assert torch.equal(dlt, torch.from_numpy(want_d).cuda()), "quant_predict"
     assert li == ls and torch.equal(cs2[:li], cs[:ls]), "hom_sum_i32 and hom_sum_f32 differ"
     del dlt, want_d
-    if full_oracle:
-        want_b = orc.compress(yh, eb)
-        pt.same(cb, lb, want_b, "compress (second operand)")
-        pt.same(cs2, ls2, orc.hom_add(want_a, want_b, n), "hom_add")
     want_dec = orc.decompress(want_s, n, eb)
     assert torch.equal(dec.view(torch.int32), torch.from_numpy(want_dec.view(np.int32)).cuda()), "decompressed sum"
     if properties:
