@@ -30,8 +30,16 @@ def test_host_helpers(pkg, orc):
         assert pkg.header_bytes(n) == orc.header_bytes(n)
         assert pkg.max_stream_bytes(n) == orc.max_stream_bytes(n)
         assert pkg.ref_cmpsize(12345, n) == 12345 + orc.header_bytes(n)
+        # one tile offset per 4096 elements of the length padded to 32768 (8 tiles per chunk of the reference)
+        assert pkg.tile_offsets_count(n) == orc.padded_len(n) // 4096 == 8 * (orc.header_bytes(n) // 1024)
     assert pkg.status_string(0) == "ok"
     assert pkg.status_string(-3).startswith("nbEle")
+    # entry points that take a workspace refuse a null one before they touch the GPU
+    L = pkg.lib()
+    assert L.homcomp_workspace_tile_offsets(None, None, None, None) == -1
+    assert L.homcomp_workspace_last_launch(None, None, None) == -1
+    assert L.homcomp_workspace_set_option(None, pkg.OPT_LDS_BUDGET, 0) == -1
+    assert L.homcomp_workspace_destroy(None) == 0
     import numpy as np
     assert np.float32(pkg.rel_to_abs(1e-4, -3.5, 4.25)) == orc.rel_to_abs(1e-4, -3.5, 4.25)
 
