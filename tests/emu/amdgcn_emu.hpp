@@ -1,0 +1,384 @@
+// TEST INFRASTRUCTURE: a host-side execution model for the device code of the HomComp kernels.
+//
+// The kernels under tirocinio-triennale_amd/csrc are written against wave64 primitives (DPP lane
+// permutations, ballots, readlane, byte permutes, range-checked buffer accesses, LDS shared by a
+// workgroup, device-scope words other workgroups poll).  This header gives those primitives a
+// plain C++ meaning so that the same source text runs on the CPU:
+//
+//   lane        one OS thread; a wave is 64 of them, a workgroup 256 in one process
+//   workgroup   one process (forked by the driver): `__shared__` becomes `static`, so every
+//               process has its own copy, like every workgroup its own LDS
+//   device      memory: one shared anonymous mapping created before the fork, same addresses in
+//               every process; device-scope atomics are host atomics on it
+//   cross-lane  operations: the lanes of a wave meet at a barrier, exchange through a slot array
+//               and go on (all of them must execute the operation, as on the hardware all lanes
+//               must be active for DPP); wave_lds_fence is a real wave barrier here, because the
+//               lanes do not run in lockstep
+//
+// It models what the instruction set defines (lane sources of the DPP controls, byte selectors of
+// v_perm, field extracts, saturating conversion, zero for loads and nothing for stores beyond a
+// buffer descriptor's byte count).  It does not model timing, register allocation or the
+// compiler: it checks the kernels' logic and their address arithmetic, not their code generation.
+// Nothing under tirocinio-triennale_amd/ includes this file.
+#pragma once
+
+#include <pthread.h>
+#include <sched.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <cmath>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline __attribute__((always_inline))
+#define __launch_bounds__(...)
+#define __shared__ static
+#define __align__(n) __attribute__((aligned(n)))
+#define amdgpu_waves_per_eu(n) unused
+
+// ---------------------------------------------------------------- thread identity
+struct emu_dim3 {
+    unsigned x = 1, y = 1, z = 1;
+};
+typedef emu_dim3 dim3;
+extern thread_local emu_dim3 threadIdx;
+extern emu_dim3 blockIdx, gridDim, blockDim;   // one workgroup per process
+
+// A byte store whose place in the wave's instruction stream matters (see emu_ordered_store8).
+struct emu_store {
+    uint8_t *addr;
+    uint32_t seq;
+    uint8_t value;
+};
+struct emu_wave {
+    pthread_barrier_t bar;
+    uint64_t slot[2][64];
+    uint8_t dirty[2][64];
+    std::vector<emu_store> log[64];
+};
+extern thread_local emu_wave *emu_wave_of_thread;
+extern thread_local int emu_lane;
+extern thread_local unsigned emu_parity;
+extern pthread_barrier_t emu_block_barrier;
+
+// Every access a kernel makes to "device memory" must fall into a registered allocation; the
+// first one that does not is reported with its address and aborts the run.
+struct emu_alloc {
+    uintptr_t lo, hi;
+    const char *name;
+};
+extern emu_alloc emu_allocs[64];
+extern int emu_n_allocs;
+inline void emu_check(const void *p, size_t bytes, const char *what)
+{
+    const uintptr_t a = (uintptr_t)p;
+    for (int i = 0; i < emu_n_allocs; ++i)
+        if (a >= emu_allocs[i].lo && a + bytes <= emu_allocs[i].hi) return;
+    fprintf(stderr, "EMU: %s of %zu bytes at %p is outside every buffer (block %u thread %u)\n", what, bytes, p, blockIdx.x,
+            threadIdx.x);
+    for (int i = 0; i < emu_n_allocs; ++i)
+        fprintf(stderr, "   %-12s [%p, %p)\n", emu_allocs[i].name, (void *)emu_allocs[i].lo, (void *)emu_allocs[i].hi);
+    fflush(stderr);
+    abort();
+}
+
+// Stores in instruction order.  On the hardware the lanes of a wave execute one instruction
+// together, so of two stores to one address the one later in the program wins, whichever lanes
+// issue them; the encoder's back end relies on that (a lane also writes bytes for planes its
+// block does not have, and a later instruction of another lane overwrites them).  Lanes that are
+// threads have no such order, so these stores are logged with their position in the program
+// (`seq`: the count of calls of the storing function so far, which is the same in all lanes, and
+// the store's index inside it) and carried out in that order at the wave's next meeting point.
+extern thread_local uint32_t emu_call_seq;
+extern thread_local bool emu_dirty;
+inline void emu_ordered_enter() { emu_call_seq += 64; }
+inline void emu_ordered_store8(uint8_t *addr, uint8_t value, uint32_t index)
+{
+    emu_wave_of_thread->log[emu_lane].push_back(emu_store{addr, emu_call_seq + index, value});
+    emu_dirty = true;
+}
+inline void emu_ordered_store(void *addr, const void *value, uint32_t bytes, uint32_t index)
+{
+    for (uint32_t i = 0; i < bytes; ++i) emu_ordered_store8((uint8_t *)addr + i, ((const uint8_t *)value)[i], index);
+}
+inline void emu_ordered_store32(void *addr, uint32_t value, uint32_t index) { emu_ordered_store(addr, &value, 4, index); }
+// after the barrier of a meeting: carries out the logged stores if any lane has some
+inline void emu_flush_stores(emu_wave *w, unsigned p)
+{
+    bool any = false;
+    for (int l = 0; l < 64; ++l) any |= w->dirty[p][l] != 0;
+    if (!any) return;
+    if (emu_lane == 0) {
+        std::vector<emu_store> all;
+        for (int l = 0; l < 64; ++l) {
+            all.insert(all.end(), w->log[l].begin(), w->log[l].end());
+            w->log[l].clear();
+        }
+        std::stable_sort(all.begin(), all.end(), [](const emu_store &a, const emu_store &b) { return a.seq < b.seq; });
+        for (const emu_store &st : all) *st.addr = st.value;
+    }
+    emu_dirty = false;
+    pthread_barrier_wait(&w->bar);
+}
+// all lanes of the wave meet; each leaves a value and reads another lane's (src < 0: none, gives 0)
+inline uint64_t emu_exchange(uint64_t mine, int src)
+{
+    emu_wave *w = emu_wave_of_thread;
+    const unsigned p = emu_parity & 1u;
+    emu_parity++;
+    w->slot[p][emu_lane] = mine;
+    w->dirty[p][emu_lane] = emu_dirty;
+    pthread_barrier_wait(&w->bar);
+    const uint64_t got = src >= 0 ? w->slot[p][src] : 0;
+    emu_flush_stores(w, p);
+    return got;
+}
+// the same, every lane seeing all values (valid until the lane's next meeting but one)
+inline const uint64_t *emu_gather(uint64_t mine)
+{
+    emu_wave *w = emu_wave_of_thread;
+    const unsigned p = emu_parity & 1u;
+    emu_parity++;
+    w->slot[p][emu_lane] = mine;
+    w->dirty[p][emu_lane] = emu_dirty;
+    pthread_barrier_wait(&w->bar);
+    emu_flush_stores(w, p);
+    return w->slot[p];
+}
+
+inline void __syncthreads() { pthread_barrier_wait(&emu_block_barrier); }
+
+// ---------------------------------------------------------------- cross-lane builtins
+// v_mov_b32 with a DPP control (the controls the kernels use): the lane the value comes from,
+// or -1 when the control names no lane for this one.
+inline int emu_dpp_source(int lane, int ctrl)
+{
+    const int row = lane & ~15, in_row = lane & 15;
+    if (ctrl >= 0x000 && ctrl <= 0x0ff) return (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3);   // quad_perm
+    if (ctrl >= 0x101 && ctrl <= 0x10f) return in_row + (ctrl & 15) <= 15 ? lane + (ctrl & 15) : -1;   // row_shl
+    if (ctrl >= 0x111 && ctrl <= 0x11f) return in_row >= (ctrl & 15) ? lane - (ctrl & 15) : -1;        // row_shr
+    if (ctrl == 0x140) return row | (15 - in_row);                                                    // row_mirror
+    if (ctrl == 0x141) return (lane & ~7) | (7 - (lane & 7));                                         // row_half_mirror
+    if (ctrl == 0x142) return lane >= 16 ? (row - 16) | 15 : -1;                                      // row_bcast:15
+    if (ctrl == 0x143) return lane >= 32 ? 31 : -1;                                                   // row_bcast:31
+    fprintf(stderr, "EMU: DPP control 0x%x is not modelled\n", ctrl);
+    abort();
+}
+inline int emu_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl)
+{
+    const int lane = emu_lane;
+    const int from = emu_dpp_source(lane, ctrl);
+    const uint64_t got = emu_exchange((uint32_t)src, from);
+    const bool enabled = ((row_mask >> (lane >> 4)) & 1) && ((bank_mask >> ((lane >> 2) & 3)) & 1);
+    if (!enabled) return old;
+    // row_bcast writes only the lanes it has a source for; the others keep `old`
+    if (from < 0) return (bound_ctrl && ctrl != 0x142 && ctrl != 0x143) ? 0 : old;
+    return (int)(uint32_t)got;
+}
+inline int emu_readfirstlane(int v) { return (int)(uint32_t)emu_exchange((uint32_t)v, 0); }
+inline int emu_readlane(int v, int lane) { return (int)(uint32_t)emu_exchange((uint32_t)v, lane & 63); }
+inline uint64_t emu_ballot(bool pred)
+{
+    const uint64_t *all = emu_gather(pred ? 1u : 0u);
+    uint64_t m = 0;
+    for (int l = 0; l < 64; ++l) m |= (all[l] & 1u) << l;
+    return m;
+}
+template <typename T>
+inline T __shfl_xor(T v, int mask, int /*width*/)
+{
+    static_assert(sizeof(T) == 4, "32-bit values");
+    uint32_t bits;
+    memcpy(&bits, &v, 4);
+    const uint32_t got = (uint32_t)emu_exchange(bits, (emu_lane ^ mask) & 63);
+    T out;
+    memcpy(&out, &got, 4);
+    return out;
+}
+inline void emu_wave_barrier() { (void)emu_exchange(0, -1); }
+
+// ---------------------------------------------------------------- lane-local builtins
+inline uint32_t emu_perm(uint32_t s0, uint32_t s1, uint32_t sel)
+{
+    // v_perm_b32: selector bytes 0-3 pick bytes of the second operand, 4-7 of the first, 0x0c gives 0x00, 0x0d and up 0xff
+    const uint64_t both = ((uint64_t)s0 << 32) | s1;
+    uint32_t out = 0;
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t c = (sel >> (8 * i)) & 0xffu;
+        uint32_t b;
+        if (c <= 7) b = (uint32_t)(both >> (8 * c)) & 0xffu;
+        else if (c == 0x0c) b = 0;
+        else if (c >= 0x0d) b = 0xff;
+        else {   // 8..11: the sign of a byte, replicated
+            const uint32_t byte = (uint32_t)(both >> (8 * (2 * (c - 8) + 1))) & 0xffu;
+            b = (byte & 0x80u) ? 0xffu : 0u;
+        }
+        out |= b << (8 * i);
+    }
+    return out;
+}
+inline uint32_t emu_alignbit(uint32_t hi, uint32_t lo, uint32_t sh) { return (uint32_t)((((uint64_t)hi << 32) | lo) >> (sh & 31u)); }
+inline uint32_t emu_alignbyte(uint32_t hi, uint32_t lo, uint32_t sh) { return (uint32_t)((((uint64_t)hi << 32) | lo) >> (8u * (sh & 3u))); }
+inline uint32_t emu_ubfe(uint32_t v, uint32_t off, uint32_t width)
+{
+    off &= 31u;
+    width &= 31u;
+    return width ? (v >> off) & ((1u << width) - 1u) : 0u;
+}
+inline int32_t emu_sbfe(int32_t v, uint32_t off, uint32_t width)
+{
+    off &= 31u;
+    width &= 31u;
+    if (!width) return 0;
+    const uint32_t field = ((uint32_t)v >> off) & ((1u << width) - 1u);
+    return (field >> (width - 1)) & 1u ? (int32_t)(field | ~((1u << width) - 1u)) : (int32_t)field;
+}
+inline uint32_t emu_sad_u8(uint32_t a, uint32_t b, uint32_t acc)
+{
+    for (int i = 0; i < 4; ++i) {
+        const int x = (a >> (8 * i)) & 0xff, y = (b >> (8 * i)) & 0xff;
+        acc += (uint32_t)(x > y ? x - y : y - x);
+    }
+    return acc;
+}
+// v_cvt_i32_f32: toward zero, saturating, NaN gives 0
+inline int32_t emu_cvt_i32_f32(float t)
+{
+    if (std::isnan(t)) return 0;
+    if (t >= 2147483648.0f) return INT32_MAX;
+    if (t <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)t;
+}
+inline int __clz(int v) { return v ? __builtin_clz((unsigned)v) : 32; }
+inline float __fmul_rn(float a, float b) { volatile float r = a * b; return r; }
+inline float __fadd_rn(float a, float b) { volatile float r = a + b; return r; }
+
+// ---------------------------------------------------------------- buffer descriptors
+struct emu_rsrc {
+    uint8_t *base;
+    uint32_t bytes;
+};
+typedef unsigned int emu_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int emu_u32x2 __attribute__((ext_vector_type(2)));
+inline emu_rsrc emu_make_rsrc(void *base, short /*stride*/, int bytes, int /*flags*/) { return emu_rsrc{(uint8_t *)base, (uint32_t)bytes}; }
+// dword d of an access at `off` is in range when it ends within the descriptor's byte count
+template <int DWORDS>
+inline void emu_buf_load(const emu_rsrc &rs, uint32_t voff, uint32_t soff, uint32_t *out)
+{
+    const uint64_t off = (uint64_t)voff + soff;
+    for (int d = 0; d < DWORDS; ++d) {
+        out[d] = 0;
+        if (off + 4u * d + 4u <= rs.bytes) {
+            emu_check(rs.base + off + 4u * d, 4, "buffer load");
+            memcpy(&out[d], rs.base + off + 4u * d, 4);
+        } else if (off + 4u * d < rs.bytes) {   // a dword that straddles the end: the bytes below it
+            const uint32_t n = (uint32_t)(rs.bytes - (off + 4u * d));
+            emu_check(rs.base + off + 4u * d, n, "buffer load");
+            memcpy(&out[d], rs.base + off + 4u * d, n);
+        }
+    }
+}
+template <int DWORDS>
+inline void emu_buf_store(const emu_rsrc &rs, uint32_t voff, uint32_t soff, const uint32_t *in)
+{
+    const uint64_t off = (uint64_t)voff + soff;
+    for (int d = 0; d < DWORDS; ++d)
+        if (off + 4u * d + 4u <= rs.bytes) {
+            emu_check(rs.base + off + 4u * d, 4, "buffer store");
+            memcpy(rs.base + off + 4u * d, &in[d], 4);
+        }
+}
+inline emu_u32x4 emu_load_b128(emu_rsrc rs, int voff, int soff, int)
+{
+    uint32_t w[4];
+    emu_buf_load<4>(rs, (uint32_t)voff, (uint32_t)soff, w);
+    return emu_u32x4{w[0], w[1], w[2], w[3]};
+}
+inline emu_u32x2 emu_load_b64(emu_rsrc rs, int voff, int soff, int)
+{
+    uint32_t w[2];
+    emu_buf_load<2>(rs, (uint32_t)voff, (uint32_t)soff, w);
+    return emu_u32x2{w[0], w[1]};
+}
+inline uint32_t emu_load_b32(emu_rsrc rs, int voff, int soff, int)
+{
+    uint32_t w;
+    emu_buf_load<1>(rs, (uint32_t)voff, (uint32_t)soff, &w);
+    return w;
+}
+inline uint16_t emu_load_b16(emu_rsrc rs, int voff, int soff, int)
+{
+    const uint64_t off = (uint64_t)(uint32_t)voff + (uint32_t)soff;
+    uint16_t v = 0;
+    if (off + 2u <= rs.bytes) {
+        emu_check(rs.base + off, 2, "buffer load");
+        memcpy(&v, rs.base + off, 2);
+    }
+    return v;
+}
+inline void emu_store_b128(emu_u32x4 v, emu_rsrc rs, int voff, int soff, int)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    emu_buf_store<4>(rs, (uint32_t)voff, (uint32_t)soff, w);
+}
+inline void emu_store_b64(emu_u32x2 v, emu_rsrc rs, int voff, int soff, int)
+{
+    const uint32_t w[2] = {v.x, v.y};
+    emu_buf_store<2>(rs, (uint32_t)voff, (uint32_t)soff, w);
+}
+inline void emu_store_b8(uint8_t v, emu_rsrc rs, int voff, int soff, int)
+{
+    const uint64_t off = (uint64_t)(uint32_t)voff + (uint32_t)soff;
+    if (off + 1u <= rs.bytes) {
+        emu_check(rs.base + off, 1, "buffer store");
+        rs.base[off] = v;
+    }
+}
+
+#define __amdgpu_buffer_rsrc_t emu_rsrc
+#define __builtin_amdgcn_make_buffer_rsrc emu_make_rsrc
+#define __builtin_amdgcn_raw_buffer_load_b128 emu_load_b128
+#define __builtin_amdgcn_raw_buffer_load_b64 emu_load_b64
+#define __builtin_amdgcn_raw_buffer_load_b32 emu_load_b32
+#define __builtin_amdgcn_raw_buffer_load_b16 emu_load_b16
+#define __builtin_amdgcn_raw_buffer_store_b128 emu_store_b128
+#define __builtin_amdgcn_raw_buffer_store_b64 emu_store_b64
+#define __builtin_amdgcn_raw_buffer_store_b8 emu_store_b8
+#define __builtin_amdgcn_update_dpp emu_update_dpp
+#define __builtin_amdgcn_readfirstlane emu_readfirstlane
+#define __builtin_amdgcn_readlane emu_readlane
+#define __builtin_amdgcn_ballot_w64 emu_ballot
+#define __builtin_amdgcn_perm emu_perm
+#define __builtin_amdgcn_alignbit emu_alignbit
+#define __builtin_amdgcn_alignbyte emu_alignbyte
+#define __builtin_amdgcn_ubfe emu_ubfe
+#define __builtin_amdgcn_sbfe emu_sbfe
+#define __builtin_amdgcn_sad_u8 emu_sad_u8
+#define __builtin_amdgcn_s_sleep(n) sched_yield()
+#define __builtin_amdgcn_s_setprio(n) ((void)0)
+#define __builtin_amdgcn_fence(order, scope) __atomic_thread_fence(__ATOMIC_SEQ_CST)
+#define __builtin_amdgcn_wave_barrier emu_wave_barrier
+
+// device-scope atomics: host atomics on the shared mapping
+#define __HIP_MEMORY_SCOPE_AGENT 0
+#define __hip_atomic_load(p, order, scope) __atomic_load_n((p), __ATOMIC_SEQ_CST)
+#define __hip_atomic_store(p, v, order, scope) __atomic_store_n((p), (v), __ATOMIC_SEQ_CST)
+inline unsigned atomicOr(uint32_t *p, uint32_t v) { return __atomic_fetch_or(p, v, __ATOMIC_SEQ_CST); }
+
+// ---------------------------------------------------------------- HIP host types the launch interface names
+typedef int hipError_t;
+typedef void *hipStream_t;
+constexpr hipError_t hipSuccess = 0, hipErrorInvalidValue = 1;
+struct float4 {
+    float x, y, z, w;
+};
+struct int4 {
+    int x, y, z, w;
+};
+inline int4 make_int4(int x, int y, int z, int w) { return int4{x, y, z, w}; }

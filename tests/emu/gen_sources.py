@@ -1,0 +1,96 @@
+"""Copies the device code of the product into tests/emu/_gen with the few textual changes a host
+compiler needs (TEST INFRASTRUCTURE; see amdgcn_emu.hpp): inline GPU assembly becomes the C++
+it stands for, address-space qualifiers go, the dynamic LDS array gets a size, and the launchers
+(host code that needs the HIP runtime) are cut off.  Every change must apply exactly once, so a
+drift of the product source is noticed here and not as a silently untested kernel."""
+from __future__ import annotations
+
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(os.path.dirname(HERE)), "tirocinio-triennale_amd", "csrc")
+GEN = os.path.join(HERE, "_gen")
+
+DEVICE_EDITS = [
+    ('    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(t));', "    r = emu_cvt_i32_f32(t);"),
+    ('    asm("v_xad_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));', "    r = (a ^ b) + c;"),
+    ('        asm("" : "+v"(mask));', ""),
+    ('    asm("" : "+v"(carry));', ""),
+    # the encoder's byte stores, whose order across the lanes of a wave matters (emu_ordered_store8):
+    # positions 0-31 the planes from the highest down, 32 the sign byte, 33 the outlier byte
+    ("        stage[base + 4u * (uint32_t)(8 * G + r)] = (uint8_t)((r < 4 ? lo : hi) >> (8 * (r & 3)));",
+     "        emu_ordered_store8(&stage[base + 4u * (uint32_t)(8 * G + r)], (uint8_t)((r < 4 ? lo : hi) >> (8 * (r & 3))), 8 * (3 - G) + (7 - r));"),
+    ("    for (int r = 3; r >= 0; --r) stage[base + 4u * (uint32_t)r] = (uint8_t)(y >> (8 * r));",
+     "    for (int r = 3; r >= 0; --r) emu_ordered_store8(&stage[base + 4u * (uint32_t)r], (uint8_t)(y >> (8 * r)), 28 + (3 - r));"),
+    ("    const bool low = __builtin_amdgcn_ballot_w64((hdr & 0x1fu) > 4u) == 0;\n    if (hdr == 0) return;",
+     "    const bool low = __builtin_amdgcn_ballot_w64((hdr & 0x1fu) > 4u) == 0;\n    emu_ordered_enter();\n    if (hdr == 0) return;"),
+    ("    stage[pos0 + ob + (uint32_t)k] = (uint8_t)sb; ", "    emu_ordered_store8(&stage[pos0 + ob + (uint32_t)k], (uint8_t)sb, 32); "),
+    ("    if ((uint32_t)k < ob) stage[pos0 + (uint32_t)k] = (uint8_t)(a0 >> (8 * k)); ",
+     "    if ((uint32_t)k < ob) emu_ordered_store8(&stage[pos0 + (uint32_t)k], (uint8_t)(a0 >> (8 * k)), 33); "),
+    # the same for the writer of wide blocks, whose 16-byte pieces reach up to 12 bytes into the next block:
+    # positions 0-5 the pieces from the highest down, then the outlier word, the sign word, words 1 to 3
+    ("                *(__attribute__((address_space(3))) u32x4_unaligned *)(at + 16u * j) =\n                    u32x4{o.w[4 * j], o.w[4 * j + 1], o.w[4 * j + 2], o.w[4 * j + 3]};",
+     "                emu_ordered_store(at + 16u * j, &o.w[4 * j], 16, kWideChunks - j);"),
+    ("    if (o.ob) store_u32_any(stage + pos, o.a0);\n    store_u32_any(at, o.w[0]);",
+     "    if (o.ob) emu_ordered_store32(stage + pos, o.a0, kWideChunks);\n    emu_ordered_store32(at, o.w[0], kWideChunks + 1);"),
+    ("        if (w <= o.F) store_u32_any(at + 4u * w, o.w[w]);", "        if (w <= o.F) emu_ordered_store32(at + 4u * w, o.w[w], kWideChunks + 1 + w);"),
+]
+KERNEL_EDITS = [
+    ("    extern __shared__ __align__(16) uint8_t s_dyn[];", "    static __attribute__((aligned(16))) uint8_t s_dyn[EMU_DYN_LDS];"),
+    ('            if constexpr (kSlicedLocal) asm volatile("" : "+v"(fresh_lane));', ""),
+    # A wave's LDS instructions take effect in the order of the program, for all its lanes: what the lanes packed is
+    # in the stage when the instructions that move it elsewhere read it.  Lanes that are threads have to meet for that.
+    ("            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {\n",
+     "            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {\n                emu_wave_barrier();\n"),
+]
+LAUNCHERS = "// ---------------------------------------------------------------- launchers"
+
+
+def edit(text: str, edits, what: str) -> str:
+    for old, new in edits:
+        if text.count(old) != 1:
+            raise SystemExit(f"gen_sources: expected exactly one occurrence in {what} of: {old!r}")
+        text = text.replace(old, new)
+    for space in ("__attribute__((address_space(3))) ", "__attribute__((address_space(1))) "):
+        text = text.replace(space, "")
+    if "address_space" in text or "asm(" in text.replace('asm volatile("" ::: "memory")', ""):
+        raise SystemExit(f"gen_sources: {what} still holds GPU-only constructs")
+    return text
+
+
+def main() -> None:
+    os.makedirs(GEN, exist_ok=True)
+    dev = edit(open(os.path.join(CSRC, "homcomp_device.hpp")).read(), DEVICE_EDITS, "homcomp_device.hpp")
+    ker = open(os.path.join(CSRC, "homcomp_kernels.hip")).read()
+    if ker.count(LAUNCHERS) != 1:
+        raise SystemExit("gen_sources: the launchers marker moved")
+    ker = ker[:ker.index(LAUNCHERS)] + "}  // namespace hc\n"
+    ker = edit(ker, KERNEL_EDITS, "homcomp_kernels.hip")
+    open(os.path.join(GEN, "homcomp_device.hpp"), "w").write(dev)
+    open(os.path.join(GEN, "homcomp_kernels.inc"), "w").write(ker)
+    open(os.path.join(GEN, "homcomp_kernels.hpp"), "w").write(open(os.path.join(CSRC, "homcomp_kernels.hpp")).read())
+
+
+CLANG = "/opt/rocm/lib/llvm/bin/clang++"   # the vector types and builtins of the device code need clang
+BINARY = os.path.join(GEN, "emu_main")
+
+
+def build(force: bool = False) -> str:
+    """Generates the sources and compiles the driver; returns the program's path.  Rebuilt when the
+    product's device code or a file of the execution model is newer than the program."""
+    import subprocess
+
+    inputs = [os.path.join(CSRC, f) for f in ("homcomp_device.hpp", "homcomp_kernels.hip", "homcomp_kernels.hpp")]
+    inputs += [os.path.join(HERE, f) for f in ("amdgcn_emu.hpp", "emu_main.cpp", "gen_sources.py", os.path.join("hip", "hip_runtime.h"))]
+    if not force and os.path.exists(BINARY) and all(os.path.getmtime(f) <= os.path.getmtime(BINARY) for f in inputs):
+        return BINARY
+    main()
+    # -O0: the run time is the lanes' meetings, not the arithmetic, and the compile takes seconds instead of a minute
+    subprocess.run([CLANG, "-std=c++17", "-O0", "-g", "-pthread", "-I" + HERE, "-Wno-unused-value",
+                    "-o", BINARY, os.path.join(HERE, "emu_main.cpp")], check=True)
+    return BINARY
+
+
+if __name__ == "__main__":
+    print(build(force=True))
