@@ -60,8 +60,9 @@ def pytest_unconfigure(config):
     ordinary assertion failure (the summary line `1 failed, 141 passed` was already out).  A
     process that dies that way with a GPU context open looks like a GPU fault from outside.
     Nothing a test checks happens after this point, so the status pytest arrived at is returned
-    as it is.  Sessions that never touched the GPU end the normal way."""
-    if _session["used_gpu"] and _session["exitstatus"] is not None:
+    as it is.  Sessions that never touched the GPU, and sessions in which every test passed (they
+    have always ended cleanly), end the normal way, exit handlers included."""
+    if _session["used_gpu"] and _session["exitstatus"] not in (None, 0):
         sys.stdout.flush()
         sys.stderr.flush()
         os._exit(_session["exitstatus"])
