@@ -38,7 +38,9 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
-#define __shared__ static
+// LDS: one copy per process, in a section of its own so that the driver can fill all of it with
+// a pattern before a workgroup starts (the hardware hands a workgroup whatever the last one left)
+#define __shared__ static __attribute__((section("emu_lds")))
 #define __align__(n) __attribute__((aligned(n)))
 #define amdgpu_waves_per_eu(n) unused
 

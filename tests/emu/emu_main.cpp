@@ -114,9 +114,13 @@ void *lane_main(void *arg)
     return nullptr;
 }
 
+extern "C" uint8_t __start_emu_lds[], __stop_emu_lds[];   // the section of the `__shared__` arrays
+
 // One workgroup of `threads` lanes in this (forked) process.
 void run_block(const Launch &l, unsigned threads)
 {
+    // LDS as the workgroup finds it: not zeros
+    for (uint8_t *b = __start_emu_lds; b != __stop_emu_lds; ++b) *b = (uint8_t)(0xC3u ^ (uintptr_t)b * 37u ^ blockIdx.x * 11u);
     const unsigned waves = (threads + 63) / 64;
     std::vector<emu_wave> w(waves);
     for (unsigned i = 0; i < waves; ++i) pthread_barrier_init(&w[i].bar, nullptr, 64);
@@ -293,7 +297,13 @@ int main(int argc, char **argv)
     p.sliced = kind;
     p.plain = plain;
     p.stage_bytes = budget;
+    // What an earlier call on the same workspace leaves behind: status words of the epoch before
+    // (totals and prefixes that look finished but are not this call's), a used spill area, old offsets.
+    auto stale_words = [](uint64_t *w, size_t count, uint32_t epoch) {
+        for (size_t i = 0; i < count; ++i) w[i] = hc::status_word(epoch, 1u + (uint32_t)(i & 1u), 0x123456789ull * (i + 1));
+    };
     uint64_t *words = (uint64_t *)device_alloc(2 * (size_t)n_tiles * 8, "scan words");
+    stale_words(words, 2 * (size_t)n_tiles, p.epoch - 1);
     p.tile_totals = words;
     p.tile_prefixes = words + n_tiles;
     uint64_t *misc = (uint64_t *)device_alloc(64, "length+error");
@@ -301,6 +311,7 @@ int main(int argc, char **argv)
     p.error = (uint32_t *)(misc + 1);
     if (enc) {
         p.spill = device_alloc((size_t)groups * 4 * slots * hc::kSpillSlotBytes, "spill area");
+        memset(p.spill, 0xD7, (size_t)groups * 4 * slots * hc::kSpillSlotBytes);
         p.out_cmp = device_alloc(cap, "out stream", 1);
         memset(p.out_cmp, 0xA5, cap);
         if (ofs_path) {
@@ -341,7 +352,9 @@ int main(int argc, char **argv)
         for (int c = 0; c < n_in; ++c) {
             oc.a.hdr[c] = p.in[c];
             oc.a.block_words[c] = (uint64_t *)device_alloc((size_t)(n_tiles / 256 + 1) * 8, "pre-pass words");
+            stale_words(oc.a.block_words[c], n_tiles / 256 + 1, p.epoch - 1);
             oc.a.ofs[c] = (uint64_t *)device_alloc((size_t)n_tiles * 8, "tile offsets in");
+            memset(oc.a.ofs[c], 0xEE, (size_t)n_tiles * 8);
             p.in_ofs[c] = oc.a.ofs[c];
         }
         oc.a.few_limit = local ? hc::kFewPlanes : hc::kSlicedMaxF;
