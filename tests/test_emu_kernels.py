@@ -192,6 +192,37 @@ def test_stated_size_cuts_the_stream_short(emu, orc, gen, name):
                  f"{what} hom_add kind {kind}")
 
 
+@pytest.mark.parametrize("n", [4099, 32768 + 4096 * 5 + 21])
+@pytest.mark.parametrize("name", ["smooth_coarse", "smooth_fine", "any_bits"])
+def test_stated_size_is_the_buffers_capacity(emu, orc, gen, name, n):
+    """The ring with its lengths on the device states every incoming stream's size as the capacity of
+    the buffer it arrived in: the stream is followed by whatever the buffer held before, and every
+    block is active.  The integer deltas come from quant_predict, as in that schedule
+    (HomComp/src/cuda_awareallreduce.cu:212-235)."""
+    x, y, eb, _ = operands(gen, orc, name, n)
+    ca, cb = orc.compress(x, eb), orc.compress(y, eb)
+    cap = orc.max_stream_bytes(n)
+    rng = np.random.default_rng(3)
+    buf_a = rng.integers(0, 256, cap, dtype=np.uint8)
+    buf_a[:ca.size] = ca
+    buf_b = rng.integers(0, 256, cap, dtype=np.uint8)
+    buf_b[:cb.size] = cb
+    same_f32(emu.run("decompress", n, eb, buf_a, dtype=np.float32), orc.decompress(buf_a, n, eb, cmp_size=cap), "decompress")
+    deltas = emu.run("quant_predict", n, eb, y, dtype=np.int32)
+    assert np.array_equal(deltas, orc.quant_predict(y, eb)), "quant_predict"
+    # (the two sums differ in the block that holds the end of a ragged operand: the float path's first
+    # padded element has the delta 0 - q[n-1], the precomputed deltas end with zeros)
+    want = orc.hom_sum_i32(buf_a, deltas, cmp_in_size=cap)
+    want_f32 = orc.hom_sum_f32(buf_a, y, eb, cmp_in_size=cap)
+    for kind in (0, 1):
+        for groups, budget, slots in ((1, Emu.BUDGETS[1], 2), (3, Emu.BUDGETS[3], 3)):
+            cfg = dict(kind=kind, groups=groups, budget=budget, slots=slots)
+            same(emu.run("hom_sum_i32", n, eb, buf_a, deltas, **cfg), want, f"hom_sum_i32 kind {kind} {groups}/{budget}/{slots}")
+            same(emu.run("hom_sum_f32", n, eb, buf_a, y, **cfg), want_f32, f"hom_sum_f32 kind {kind} {groups}/{budget}/{slots}")
+    for kind in (1, 2):
+        same(emu.run("hom_add", n, eb, buf_a, buf_b, kind=kind), orc.hom_add(buf_a, buf_b, n, size_a=cap, size_b=cap), f"hom_add kind {kind}")
+
+
 def test_partial_sums_of_a_ring(emu, orc, gen):
     """Eight operands summed one after the other, the way a ring's reduce-scatter does: the plane
     counts grow with every step, so the later steps leave the few-plane path tile by tile."""
