@@ -28,6 +28,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include <algorithm>
 #include <cmath>
@@ -46,7 +47,8 @@
 
 // ---------------------------------------------------------------- thread identity
 struct emu_dim3 {
-    unsigned x = 1, y = 1, z = 1;
+    unsigned x, y, z;
+    emu_dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
 };
 typedef emu_dim3 dim3;
 extern thread_local emu_dim3 threadIdx;
@@ -74,8 +76,10 @@ extern pthread_barrier_t emu_block_barrier;
 struct emu_alloc {
     uintptr_t lo, hi;
     const char *name;
+    uintptr_t map;      // the mapping around it (guard pages included), for its release
+    size_t map_bytes;
 };
-extern emu_alloc emu_allocs[64];
+extern emu_alloc emu_allocs[256];
 extern int emu_n_allocs;
 inline void emu_check(const void *p, size_t bytes, const char *what)
 {
@@ -362,7 +366,15 @@ inline void emu_store_b8(uint8_t v, emu_rsrc rs, int voff, int soff, int)
 #define __builtin_amdgcn_ubfe emu_ubfe
 #define __builtin_amdgcn_sbfe emu_sbfe
 #define __builtin_amdgcn_sad_u8 emu_sad_u8
-#define __builtin_amdgcn_s_sleep(n) sched_yield()
+// A wave that sleeps between two looks at a word another workgroup writes: the bounds on such waits
+// count looks, and are sized for a device on which every workgroup runs at once; here a
+// workgroup may have to wait for a processor, so a look takes its time
+inline void emu_sleep()
+{
+    const timespec t{0, 20000};
+    nanosleep(&t, nullptr);
+}
+#define __builtin_amdgcn_s_sleep(n) emu_sleep()
 #define __builtin_amdgcn_s_setprio(n) ((void)0)
 #define __builtin_amdgcn_fence(order, scope) __atomic_thread_fence(__ATOMIC_SEQ_CST)
 #define __builtin_amdgcn_wave_barrier emu_wave_barrier
@@ -373,10 +385,7 @@ inline void emu_store_b8(uint8_t v, emu_rsrc rs, int voff, int soff, int)
 #define __hip_atomic_store(p, v, order, scope) __atomic_store_n((p), (v), __ATOMIC_SEQ_CST)
 inline unsigned atomicOr(uint32_t *p, uint32_t v) { return __atomic_fetch_or(p, v, __ATOMIC_SEQ_CST); }
 
-// ---------------------------------------------------------------- HIP host types the launch interface names
-typedef int hipError_t;
-typedef void *hipStream_t;
-constexpr hipError_t hipSuccess = 0, hipErrorInvalidValue = 1;
+// ---------------------------------------------------------------- vector types of the HIP headers
 struct float4 {
     float x, y, z, w;
 };

@@ -22,46 +22,26 @@
 // two inaccessible pages and ending at the upper one, so a plain access beyond a buffer is a
 // segmentation fault of the run, and every buffer-descriptor access is checked against the list
 // of buffers (emu_check).
-#include <sys/mman.h>
-#include <sys/wait.h>
-#include <unistd.h>
-
 #include <string>
 #include <vector>
 
 #define EMU_DYN_LDS (4 * 2 * (8192 + 64))
-#include "amdgcn_emu.hpp"
-
-thread_local emu_dim3 threadIdx;
-emu_dim3 blockIdx, gridDim, blockDim;
-thread_local emu_wave *emu_wave_of_thread = nullptr;
-thread_local int emu_lane = 0;
-thread_local unsigned emu_parity = 0;
-thread_local uint32_t emu_call_seq = 0;
-thread_local bool emu_dirty = false;
-pthread_barrier_t emu_block_barrier;
-emu_alloc emu_allocs[64];
-int emu_n_allocs = 0;
+#define EMU_DEFINE_GLOBALS
+#include "hip/hip_runtime.h"
 
 #include "_gen/homcomp_device.hpp"
 #include "_gen/homcomp_kernels.inc"
 
 namespace {
 
-const size_t kPage = 4096;
-
-// `bytes` of zeroed shared memory that end at an inaccessible page (and start behind one)
 uint8_t *device_alloc(size_t bytes, const char *name, size_t align = 256)
 {
-    const size_t room = (bytes + align - 1) / align * align;
-    const size_t pages = (room + kPage - 1) / kPage * kPage;
-    uint8_t *m = (uint8_t *)mmap(nullptr, pages + 2 * kPage, PROT_NONE, MAP_SHARED | MAP_ANONYMOUS, -1, 0);
-    if (m == MAP_FAILED || mprotect(m + kPage, pages, PROT_READ | PROT_WRITE) != 0) {
+    uint8_t *p = (uint8_t *)emu_device_alloc_named(bytes, name, align);
+    if (!p) {
         perror("mmap");
         exit(2);
     }
-    uint8_t *p = m + kPage + pages - room;
-    emu_allocs[emu_n_allocs++] = emu_alloc{(uintptr_t)p, (uintptr_t)p + room, name};
+    memset(p, 0, bytes);
     return p;
 }
 
@@ -97,84 +77,10 @@ struct Launch {
     const void *args;
 };
 
-struct LaneStart {
-    const Launch *launch;
-    emu_wave *wave;
-    int tid;
-};
-
-void *lane_main(void *arg)
-{
-    const LaneStart *s = (const LaneStart *)arg;
-    threadIdx.x = (unsigned)s->tid;
-    emu_lane = s->tid & 63;
-    emu_wave_of_thread = s->wave;
-    emu_parity = 0;
-    s->launch->kernel(s->launch->args);
-    return nullptr;
-}
-
-extern "C" uint8_t __start_emu_lds[], __stop_emu_lds[];   // the section of the `__shared__` arrays
-
-// One workgroup of `threads` lanes in this (forked) process.
-void run_block(const Launch &l, unsigned threads)
-{
-    // LDS as the workgroup finds it: not zeros
-    for (uint8_t *b = __start_emu_lds; b != __stop_emu_lds; ++b) *b = (uint8_t)(0xC3u ^ (uintptr_t)b * 37u ^ blockIdx.x * 11u);
-    const unsigned waves = (threads + 63) / 64;
-    std::vector<emu_wave> w(waves);
-    for (unsigned i = 0; i < waves; ++i) pthread_barrier_init(&w[i].bar, nullptr, 64);
-    pthread_barrier_init(&emu_block_barrier, nullptr, threads);
-    std::vector<pthread_t> th(threads);
-    std::vector<LaneStart> st(threads);
-    pthread_attr_t attr;
-    pthread_attr_init(&attr);
-    pthread_attr_setstacksize(&attr, 1 << 20);
-    for (unsigned t = 0; t < threads; ++t) {
-        st[t] = LaneStart{&l, &w[t / 64], (int)t};
-        if (pthread_create(&th[t], &attr, lane_main, &st[t]) != 0) {
-            perror("pthread_create");
-            _exit(3);
-        }
-    }
-    for (unsigned t = 0; t < threads; ++t) pthread_join(th[t], nullptr);
-}
-
-// A grid: one process per workgroup, all alive at the same time (the kernels' waits need that).
 void run_grid(const Launch &l, unsigned gx, unsigned gy, unsigned threads)
 {
-    gridDim.x = gx;
-    gridDim.y = gy;
-    blockDim.x = threads;
-    std::vector<pid_t> kids;
-    for (unsigned y = 0; y < gy; ++y)
-        for (unsigned x = 0; x < gx; ++x) {
-            fflush(nullptr);
-            const pid_t k = fork();
-            if (k < 0) {
-                perror("fork");
-                exit(3);
-            }
-            if (k == 0) {
-                blockIdx.x = x;
-                blockIdx.y = y;
-                run_block(l, threads);
-                fflush(nullptr);
-                _exit(0);
-            }
-            kids.push_back(k);
-        }
-    bool ok = true;
-    for (pid_t k : kids) {
-        int status = 0;
-        waitpid(k, &status, 0);
-        if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) {
-            fprintf(stderr, "EMU: a workgroup ended abnormally (status 0x%x%s)\n", status,
-                    WIFSIGNALED(status) && WTERMSIG(status) == SIGSEGV ? ": segmentation fault, an access beyond a buffer" : "");
-            ok = false;
-        }
-    }
-    if (!ok) exit(4);
+    const std::function<void()> body = [=]() { l.kernel(l.args); };
+    if (!emu_run_grid(body, emu_dim3(gx, gy), emu_dim3(threads))) exit(4);
 }
 
 template <int NIN, int LOCAL, int OUT, int BITPLANE>

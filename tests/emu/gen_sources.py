@@ -59,39 +59,75 @@ def edit(text: str, edits, what: str) -> str:
     return text
 
 
+API_EDITS = [
+    ('#include "../../include/homcomp.h"', '#include "homcomp.h"'),
+]
+
+
 def main() -> None:
     os.makedirs(GEN, exist_ok=True)
     dev = edit(open(os.path.join(CSRC, "homcomp_device.hpp")).read(), DEVICE_EDITS, "homcomp_device.hpp")
     ker = open(os.path.join(CSRC, "homcomp_kernels.hip")).read()
     if ker.count(LAUNCHERS) != 1:
         raise SystemExit("gen_sources: the launchers marker moved")
-    ker = ker[:ker.index(LAUNCHERS)] + "}  // namespace hc\n"
-    ker = edit(ker, KERNEL_EDITS, "homcomp_kernels.hip")
+    whole = edit(ker, KERNEL_EDITS, "homcomp_kernels.hip")
+    kernels_only = whole[:whole.index(LAUNCHERS)] + "}  // namespace hc\n"
+    api = edit(open(os.path.join(CSRC, "homcomp_api.hip")).read(), API_EDITS, "homcomp_api.hip")
     open(os.path.join(GEN, "homcomp_device.hpp"), "w").write(dev)
-    open(os.path.join(GEN, "homcomp_kernels.inc"), "w").write(ker)
+    open(os.path.join(GEN, "homcomp_kernels.inc"), "w").write(kernels_only)   # the kernels, for emu_main.cpp's own launches
+    open(os.path.join(GEN, "homcomp_kernels.cpp"), "w").write(whole)          # with the launchers, for the library
+    open(os.path.join(GEN, "homcomp_api.cpp"), "w").write(api)
     open(os.path.join(GEN, "homcomp_kernels.hpp"), "w").write(open(os.path.join(CSRC, "homcomp_kernels.hpp")).read())
 
 
 CLANG = "/opt/rocm/lib/llvm/bin/clang++"   # the vector types and builtins of the device code need clang
 BINARY = os.path.join(GEN, "emu_main")
+LIBRARY = os.path.join(GEN, "libhomcomp_emu.so")
+INCLUDE = os.path.join(os.path.dirname(os.path.dirname(HERE)), "include")
+# -O0: the run time is the lanes' meetings, not the arithmetic, and the compile takes seconds instead of a minute.
+# -ftrivial-auto-var-init=pattern: a local the code never set holds a pattern, not a convenient zero.
+CXXFLAGS = ["-std=c++17", "-O0", "-g", "-pthread", "-ftrivial-auto-var-init=pattern", "-Wno-unused-value"]
+
+
+def _inputs():
+    files = [os.path.join(CSRC, f) for f in ("homcomp_device.hpp", "homcomp_kernels.hip", "homcomp_kernels.hpp", "homcomp_api.hip")]
+    files += [os.path.join(HERE, f) for f in ("amdgcn_emu.hpp", "emu_runtime.hpp", "emu_main.cpp", "emu_library.cpp", "gen_sources.py",
+                                              os.path.join("hip", "hip_runtime.h"))]
+    return files + [os.path.join(INCLUDE, "homcomp.h")]
+
+
+def _fresh(target: str) -> bool:
+    return os.path.exists(target) and all(os.path.getmtime(f) <= os.path.getmtime(target) for f in _inputs())
 
 
 def build(force: bool = False) -> str:
-    """Generates the sources and compiles the driver; returns the program's path.  Rebuilt when the
-    product's device code or a file of the execution model is newer than the program."""
+    """Generates the sources and compiles the driver program (one operation per run, every launch
+    parameter an argument); returns its path.  Rebuilt when the product's device code or a file of
+    the execution model is newer than the program."""
     import subprocess
 
-    inputs = [os.path.join(CSRC, f) for f in ("homcomp_device.hpp", "homcomp_kernels.hip", "homcomp_kernels.hpp")]
-    inputs += [os.path.join(HERE, f) for f in ("amdgcn_emu.hpp", "emu_main.cpp", "gen_sources.py", os.path.join("hip", "hip_runtime.h"))]
-    if not force and os.path.exists(BINARY) and all(os.path.getmtime(f) <= os.path.getmtime(BINARY) for f in inputs):
+    if not force and _fresh(BINARY):
         return BINARY
     main()
-    # -O0: the run time is the lanes' meetings, not the arithmetic, and the compile takes seconds instead of a minute
-    # -ftrivial-auto-var-init=pattern: a local the code never set holds a pattern, not a convenient zero
-    subprocess.run([CLANG, "-std=c++17", "-O0", "-g", "-pthread", "-ftrivial-auto-var-init=pattern", "-I" + HERE, "-Wno-unused-value",
-                    "-o", BINARY, os.path.join(HERE, "emu_main.cpp")], check=True)
+    subprocess.run([CLANG, *CXXFLAGS, "-I" + HERE, "-o", BINARY, os.path.join(HERE, "emu_main.cpp")], check=True)
     return BINARY
+
+
+def build_library(force: bool = False) -> str:
+    """The whole library (C ABI, workspace logic, launchers, kernels) built for the host against the
+    execution model: libhomcomp_emu.so exports what libhomcomp_amd.so exports, plus the model's
+    allocator for the caller's buffers (emu_library.cpp)."""
+    import subprocess
+
+    if not force and _fresh(LIBRARY):
+        return LIBRARY
+    main()
+    subprocess.run([CLANG, *CXXFLAGS, "-fPIC", "-shared", "-x", "c++", "-I" + HERE, "-I" + GEN, "-I" + INCLUDE, "-include",
+                    os.path.join(HERE, "emu_library_config.h"), "-o", LIBRARY, os.path.join(HERE, "emu_library.cpp"),
+                    os.path.join(GEN, "homcomp_kernels.cpp"), os.path.join(GEN, "homcomp_api.cpp")], check=True)
+    return LIBRARY
 
 
 if __name__ == "__main__":
     print(build(force=True))
+    print(build_library(force=True))

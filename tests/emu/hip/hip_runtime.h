@@ -1,4 +1,4 @@
-// Stand-in for <hip/hip_runtime.h> in the host build of the kernels' logic (tests/emu): the
-// device code's include of the HIP runtime lands here.
+// Stand-in for <hip/hip_runtime.h> in the host build of the library's source (tests/emu): the
+// includes of the HIP runtime land here.
 #pragma once
-#include "../amdgcn_emu.hpp"
+#include "../emu_runtime.hpp"
