@@ -199,12 +199,12 @@ inline uint64_t emu_ballot(bool pred)
 template <typename T>
 inline T __shfl_xor(T v, int mask, int /*width*/)
 {
-    static_assert(sizeof(T) == 4, "32-bit values");
-    uint32_t bits;
-    memcpy(&bits, &v, 4);
-    const uint32_t got = (uint32_t)emu_exchange(bits, (emu_lane ^ mask) & 63);
+    static_assert(sizeof(T) <= 8, "values of up to 64 bits");
+    uint64_t bits = 0;
+    memcpy(&bits, &v, sizeof(T));
+    const uint64_t got = emu_exchange(bits, (emu_lane ^ mask) & 63);
     T out;
-    memcpy(&out, &got, 4);
+    memcpy(&out, &got, sizeof(T));
     return out;
 }
 inline void emu_wave_barrier() { (void)emu_exchange(0, -1); }

@@ -25,9 +25,18 @@
 // ---------------------------------------------------------------- device memory
 const size_t emu_page = 4096;
 
+// (the list is shared by the host threads of a program: ranks of a ring that allocate side by side)
+extern pthread_mutex_t emu_alloc_lock;
+struct emu_locked {
+    pthread_mutex_t *m;
+    explicit emu_locked(pthread_mutex_t *m_) : m(m_) { pthread_mutex_lock(m); }
+    ~emu_locked() { pthread_mutex_unlock(m); }
+};
+
 // `bytes` of shared memory that end (rounded up to `align`) at an inaccessible page and start behind one
 inline void *emu_device_alloc_named(size_t bytes, const char *name, size_t align = 256)
 {
+    const emu_locked lock(&emu_alloc_lock);
     if (emu_n_allocs >= (int)(sizeof emu_allocs / sizeof emu_allocs[0])) {
         fprintf(stderr, "EMU: too many allocations\n");
         abort();
@@ -42,6 +51,7 @@ inline void *emu_device_alloc_named(size_t bytes, const char *name, size_t align
 }
 inline bool emu_device_free(void *p)
 {
+    const emu_locked lock(&emu_alloc_lock);
     for (int i = 0; i < emu_n_allocs; ++i)
         if (emu_allocs[i].lo == (uintptr_t)p) {
             munmap((void *)emu_allocs[i].map, emu_allocs[i].map_bytes);
@@ -52,34 +62,50 @@ inline bool emu_device_free(void *p)
 }
 
 // ---------------------------------------------------------------- launches
-extern "C" uint8_t __start_emu_lds[], __stop_emu_lds[];   // the section of the `__shared__` arrays
+// the section of the `__shared__` arrays of this program or library (absent if it has none)
+extern "C" uint8_t __start_emu_lds[] __attribute__((weak)), __stop_emu_lds[] __attribute__((weak));
 
-struct emu_lane_start {
+// A worker process runs the workgroups first, first + step, ... of a grid one after the other, with
+// one set of lane threads for all of them (starting 256 threads per workgroup is what a large grid
+// of small workgroups would otherwise spend its time on).
+struct emu_worker {
     const std::function<void()> *kernel;
-    emu_wave *wave;
+    emu_wave *waves;
+    unsigned threads, first, step, blocks, grid_x;
+};
+struct emu_lane_start {
+    const emu_worker *worker;
     int tid;
 };
 inline void *emu_lane_main(void *arg)
 {
     const emu_lane_start *s = (const emu_lane_start *)arg;
+    const emu_worker *w = s->worker;
     threadIdx.x = (unsigned)s->tid;
     emu_lane = s->tid & 63;
-    emu_wave_of_thread = s->wave;
-    emu_parity = 0;
-    emu_call_seq = 0;
-    emu_dirty = false;
-    (*s->kernel)();
+    emu_wave_of_thread = &w->waves[s->tid / 64];
+    for (unsigned i = w->first; i < w->blocks; i += w->step) {
+        if (s->tid == 0) {
+            blockIdx.x = i % w->grid_x;
+            blockIdx.y = i / w->grid_x;
+            // LDS as the workgroup finds it: not zeros
+            for (uint8_t *b = __start_emu_lds; b && b != __stop_emu_lds; ++b) *b = (uint8_t)(0xC3u ^ (uintptr_t)b * 37u ^ i * 11u);
+        }
+        emu_parity = 0;
+        emu_call_seq = 0;
+        emu_dirty = false;
+        pthread_barrier_wait(&emu_block_barrier);
+        (*w->kernel)();
+        pthread_barrier_wait(&emu_block_barrier);
+    }
     return nullptr;
 }
 
-// One workgroup of `threads` lanes in this (forked) process.
-inline void emu_run_block(const std::function<void()> &kernel, unsigned threads)
+inline void emu_run_worker(emu_worker &w)
 {
-    // LDS as the workgroup finds it: not zeros
-    for (uint8_t *b = __start_emu_lds; b != __stop_emu_lds; ++b) *b = (uint8_t)(0xC3u ^ (uintptr_t)b * 37u ^ blockIdx.x * 11u);
-    const unsigned waves = (threads + 63) / 64;
-    emu_wave *w = new emu_wave[waves];
-    for (unsigned i = 0; i < waves; ++i) pthread_barrier_init(&w[i].bar, nullptr, i + 1 < waves || threads % 64 == 0 ? 64 : threads % 64);
+    const unsigned threads = w.threads, waves = (threads + 63) / 64;
+    w.waves = new emu_wave[waves];
+    for (unsigned i = 0; i < waves; ++i) pthread_barrier_init(&w.waves[i].bar, nullptr, i + 1 < waves || threads % 64 == 0 ? 64 : threads % 64);
     pthread_barrier_init(&emu_block_barrier, nullptr, threads);
     pthread_t *th = new pthread_t[threads];
     emu_lane_start *st = new emu_lane_start[threads];
@@ -87,7 +113,7 @@ inline void emu_run_block(const std::function<void()> &kernel, unsigned threads)
     pthread_attr_init(&attr);
     pthread_attr_setstacksize(&attr, 1 << 20);
     for (unsigned t = 0; t < threads; ++t) {
-        st[t] = emu_lane_start{&kernel, &w[t / 64], (int)t};
+        st[t] = emu_lane_start{&w, (int)t};
         if (pthread_create(&th[t], &attr, emu_lane_main, &st[t]) != 0) {
             perror("EMU: pthread_create");
             _exit(3);
@@ -96,33 +122,44 @@ inline void emu_run_block(const std::function<void()> &kernel, unsigned threads)
     for (unsigned t = 0; t < threads; ++t) pthread_join(th[t], nullptr);
 }
 
-// A grid: one process per workgroup, all alive at the same time (the kernels' waits need that).
+// A grid.  Up to emu_resident_limit() workgroups are alive at the same time, each in a process of
+// its own (the kernels whose workgroups wait for one another size their grids far below that).
+// The workgroups of a larger grid are dealt out to that many worker processes in turn, which run
+// theirs in index order: the unfinished workgroup with the smallest index is always running, which
+// is what a kernel may rely on (a workgroup only ever waits for workgroups with smaller indices).
 // Returns false when a workgroup ended abnormally (an access beyond a buffer, an abort of the model).
+extern pthread_mutex_t emu_launch_lock;
+inline unsigned emu_resident_limit()
+{
+    const char *e = getenv("EMU_RESIDENT");
+    const int v = e ? atoi(e) : 48;
+    return v < 1 ? 1u : (unsigned)v;
+}
 inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu_dim3 block)
 {
+    const emu_locked lock(&emu_launch_lock);   // one launch at a time, whichever host thread makes it
     gridDim = grid;
     blockDim = block;
-    const unsigned n = grid.x * grid.y * grid.z;
-    pid_t *kids = new pid_t[n];
+    const unsigned n = grid.x * grid.y * grid.z, limit = emu_resident_limit(), workers = n < limit ? n : limit;
+    pid_t *kids = new pid_t[workers];
     unsigned started = 0;
+    bool ok = true;
     fflush(nullptr);
-    for (unsigned y = 0; y < grid.y; ++y)
-        for (unsigned x = 0; x < grid.x; ++x) {
-            const pid_t k = fork();
-            if (k < 0) {
-                perror("EMU: fork");
-                break;
-            }
-            if (k == 0) {
-                blockIdx.x = x;
-                blockIdx.y = y;
-                emu_run_block(kernel, block.x);
-                fflush(nullptr);
-                _exit(0);
-            }
-            kids[started++] = k;
+    for (unsigned i = 0; i < workers; ++i) {
+        const pid_t k = fork();
+        if (k < 0) {
+            perror("EMU: fork");
+            ok = false;
+            break;
         }
-    bool ok = started == n;
+        if (k == 0) {
+            emu_worker w{&kernel, nullptr, block.x, i, workers, n, grid.x};
+            emu_run_worker(w);
+            fflush(nullptr);
+            _exit(0);
+        }
+        kids[started++] = k;
+    }
     for (unsigned i = 0; i < started; ++i) {
         int status = 0;
         waitpid(kids[i], &status, 0);
@@ -141,7 +178,8 @@ typedef int hipError_t;
 typedef void *hipStream_t;
 typedef void *hipEvent_t;
 constexpr hipError_t hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorLaunchFailure = 719;
-extern hipError_t emu_last_error;
+extern thread_local hipError_t emu_last_error;
+inline const char *hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "an error of the emulated runtime"; }
 inline hipError_t hipGetLastError()
 {
     const hipError_t e = emu_last_error;
@@ -149,10 +187,6 @@ inline hipError_t hipGetLastError()
     return e;
 }
 
-template <typename... A>
-struct emu_always_false {
-    static constexpr bool value = false;
-};
 // hipLaunchKernelGGL(kernel, grid, block, dynamic LDS, stream, arguments...)
 template <typename K, typename... A>
 inline void emu_launch(K kernel, emu_dim3 grid, emu_dim3 block, size_t dyn_lds, hipStream_t, A... args)
@@ -172,6 +206,11 @@ inline hipError_t hipMalloc(void **p, size_t bytes)
     if (*p) memset(*p, 0xB6, bytes);   // fresh device memory is not zero
     return *p ? hipSuccess : hipErrorOutOfMemory;
 }
+template <typename T>
+inline hipError_t hipMalloc(T **p, size_t bytes)
+{
+    return hipMalloc((void **)p, bytes);
+}
 inline hipError_t hipFree(void *p) { return !p || emu_device_free(p) ? hipSuccess : hipErrorInvalidValue; }
 constexpr unsigned hipHostMallocDefault = 0;
 inline hipError_t hipHostMalloc(void **p, size_t bytes, unsigned)
@@ -187,11 +226,17 @@ inline hipError_t hipMemset(void *p, int v, size_t bytes)
     return hipSuccess;
 }
 enum hipMemcpyKind { hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
-inline hipError_t hipMemcpyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind, hipStream_t)
+inline hipError_t hipMemcpy(void *dst, const void *src, size_t bytes, hipMemcpyKind kind)
 {
-    memcpy(dst, src, bytes);
+    // the side that is device memory must lie inside an allocation
+    if (kind == hipMemcpyHostToDevice || kind == hipMemcpyDeviceToDevice) emu_check(dst, bytes, "hipMemcpy (destination)");
+    if (kind == hipMemcpyDeviceToHost || kind == hipMemcpyDeviceToDevice) emu_check(src, bytes, "hipMemcpy (source)");
+    memmove(dst, src, bytes);
     return hipSuccess;
 }
+inline hipError_t hipMemcpyAsync(void *dst, const void *src, size_t bytes, hipMemcpyKind kind, hipStream_t) { return hipMemcpy(dst, src, bytes, kind); }
+inline hipError_t hipMemsetAsync(void *p, int v, size_t bytes, hipStream_t) { return hipMemset(p, v, bytes); }
+inline hipError_t hipSetDevice(int d) { return d == 0 ? hipSuccess : hipErrorInvalidValue; }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 inline hipError_t hipGetDevice(int *d)
@@ -289,5 +334,6 @@ thread_local bool emu_dirty = false;
 pthread_barrier_t emu_block_barrier;
 emu_alloc emu_allocs[256];
 int emu_n_allocs = 0;
-hipError_t emu_last_error = hipSuccess;
+thread_local hipError_t emu_last_error = hipSuccess;
+pthread_mutex_t emu_alloc_lock = PTHREAD_MUTEX_INITIALIZER, emu_launch_lock = PTHREAD_MUTEX_INITIALIZER;
 #endif

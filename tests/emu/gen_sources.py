@@ -128,6 +128,32 @@ def build_library(force: bool = False) -> str:
     return LIBRARY
 
 
+PROGRAMS = ("shim_roundtrip", "ring_allreduce", "homcomp_eval")
+
+
+def build_programs(force: bool = False) -> dict:
+    """The C++ programs of tests/cpp that drive the host-side drop-ins (GSZ_entry.hpp,
+    allreduce_ring.hpp with its ranks as host threads, homcomp_eval.hpp), built for the host
+    against the execution model and linked with libhomcomp_emu.so; returns name -> path."""
+    import subprocess
+
+    library = build_library(force)
+    host = os.path.join(os.path.dirname(CSRC), "host")
+    out = os.path.join(GEN, "cpp")
+    os.makedirs(out, exist_ok=True)
+    paths = {}
+    for name in PROGRAMS:
+        src = os.path.join(os.path.dirname(HERE), "cpp", name + ".cpp")
+        exe = paths[name] = os.path.join(out, name)
+        deps = [src, library] + [os.path.join(host, f) for f in os.listdir(host)]
+        if not force and os.path.exists(exe) and all(os.path.getmtime(f) <= os.path.getmtime(exe) for f in deps):
+            continue
+        subprocess.run([CLANG, *CXXFLAGS, "-x", "c++", "-I" + HERE, "-include", os.path.join(HERE, "emu_library_config.h"),
+                        "-o", exe, src, "-L" + GEN, "-lhomcomp_emu", "-Wl,-rpath," + GEN], check=True)
+    return paths
+
+
 if __name__ == "__main__":
     print(build(force=True))
     print(build_library(force=True))
+    print(build_programs(force=True))

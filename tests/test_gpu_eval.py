@@ -42,6 +42,12 @@ def closed_forms(ori32: np.ndarray, dec32: np.ndarray):
 def test_evaluator_report(tmp_path, orc, gen, cuda, kind, n, eb, rel):
     assert os.path.exists(EXE), "tests/cpp/homcomp_eval is not built (run __graft_entry__.build())"
     orc.set_threads(16)
+    check_evaluator_report(EXE, tmp_path, orc, gen, kind, n, eb, rel, timeout=120)
+
+
+def check_evaluator_report(exe, tmp_path, orc, gen, kind, n, eb, rel, timeout):
+    """Runs the program `exe` (the drop-in on the GPU, or its host build on the CPU execution model)
+    and checks every number it reports."""
     a = gen.GENERATORS_NP[kind](n, 1)
     b = gen.GENERATORS_NP[kind](n, 2) if kind != "smooth" else a.copy()   # the reference adds the file to itself
     if kind == "gradient_like":
@@ -50,7 +56,7 @@ def test_evaluator_report(tmp_path, orc, gen, cuda, kind, n, eb, rel):
     fa, fb, out = tmp_path / "a.f32", tmp_path / "b.f32", tmp_path / "reduced.f32"
     a.tofile(fa)
     b.tofile(fb)
-    res = subprocess.run([EXE, str(fa), str(fb), repr(eb), str(rel), str(out)], capture_output=True, text=True, timeout=120)
+    res = subprocess.run([exe, str(fa), str(fb), repr(eb), str(rel), str(out)], capture_output=True, text=True, timeout=timeout)
     assert res.returncode == 0, res.stdout + res.stderr
     kv_line = [l for l in res.stdout.splitlines() if l.startswith("KV ")][0]
     kv = dict(item.split("=") for item in kv_line.split()[1:])

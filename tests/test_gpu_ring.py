@@ -73,14 +73,20 @@ def expected(orc, data, count, eb, variant):
 def test_ring_allreduce(tmp_path, orc, gen, cuda, variant, ranks, count):
     assert os.path.exists(EXE), "tests/cpp/ring_allreduce is not built (run __graft_entry__.build())"
     orc.set_threads(16)
+    check_ring_allreduce(EXE, tmp_path, orc, gen, variant, ranks, count, timeout=100)
+
+
+def check_ring_allreduce(exe, tmp_path, orc, gen, variant, ranks, count, timeout):
+    """Runs the program `exe` (the drop-in on the GPU, or its host build on the CPU execution model)
+    and compares every rank's result with the oracle's."""
     data = [gen.smooth_np(count, 70 + r) for r in range(ranks)]
     mn, mx = orc.value_range(np.concatenate(data))
     eb = orc.rel_to_abs(1e-4, mn, mx)
     inp, outp = tmp_path / "in", tmp_path / "out"
     for r, d in enumerate(data):
         d.tofile(f"{inp}.r{r}.f32")
-    res = subprocess.run([EXE, variant, str(ranks), str(count), repr(float(eb)), str(inp), str(outp), "2"],
-                         capture_output=True, text=True, timeout=100)
+    res = subprocess.run([exe, variant, str(ranks), str(count), repr(float(eb)), str(inp), str(outp), "2"],
+                         capture_output=True, text=True, timeout=timeout)
     assert res.returncode == 0 and "status=0" in res.stdout, res.stdout + res.stderr
     want = expected(orc, data, count, eb, variant)
     for r in range(ranks):

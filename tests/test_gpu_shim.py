@@ -16,14 +16,20 @@ EXE = os.path.join(ROOT, "tests", "cpp", "shim_roundtrip")
 @pytest.mark.parametrize("n", [1 << 20, 32768 * 3 + 100])
 def test_shim_roundtrip(tmp_path, orc, gen, cuda, n):
     assert os.path.exists(EXE), "tests/cpp/shim_roundtrip is not built (run __graft_entry__.build())"
+    check_shim_roundtrip(EXE, tmp_path, orc, gen, n, timeout=120)
+
+
+def check_shim_roundtrip(exe, tmp_path, orc, gen, n, timeout):
+    """Runs the program `exe` (the drop-in on the GPU, or its host build on the CPU execution model)
+    and compares what it wrote with the oracle."""
     a, b = gen.smooth_np(n, 1), gen.smooth_np(n, 2)
     mn, mx = orc.value_range(np.concatenate([a, b]))
     eb = orc.rel_to_abs(1e-4, mn, mx)
     fa, fb, prefix = tmp_path / "a.f32", tmp_path / "b.f32", tmp_path / "out"
     a.tofile(fa)
     b.tofile(fb)
-    res = subprocess.run([EXE, str(fa), str(fb), repr(float(eb)), str(prefix)],
-                         capture_output=True, text=True, timeout=120)
+    res = subprocess.run([exe, str(fa), str(fb), repr(float(eb)), str(prefix)],
+                         capture_output=True, text=True, timeout=timeout)
     assert res.returncode == 0, res.stdout + res.stderr
     fields = dict(kv.split("=") for kv in res.stdout.split())
     want_cmp = orc.compress(a, eb)

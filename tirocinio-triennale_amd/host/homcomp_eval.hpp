@@ -178,6 +178,7 @@ inline bool error_evaluation(const float *d_ori, const float *d_dec, size_t nbEl
                                                                                             : (size_t)kEvalBlocks);
     bool ok = true;
     hipLaunchKernelGGL(k_eval_first, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_ori_b, d_dec, nbEle, scale, (EvalPartial *)d_part);
+    ok = hipGetLastError() == hipSuccess;
     ok = ok && hipMemcpyAsync(part.data(), d_part, blocks * sizeof(EvalPartial), hipMemcpyDeviceToHost, stream) == hipSuccess &&
          hipStreamSynchronize(stream) == hipSuccess;
     double sum_ori = 0, sum_dec = 0, sum_err2 = 0, max_pw = 0;
@@ -195,7 +196,7 @@ inline bool error_evaluation(const float *d_ori, const float *d_dec, size_t nbEl
     if (ok) {
         hipLaunchKernelGGL(k_eval_second, dim3(blocks), dim3(kEvalThreads), 0, stream, d_ori, d_ori_b, d_dec, nbEle, scale, mean_ori, mean_dec,
                            (EvalMoments *)d_part);
-        ok = hipMemcpyAsync(mom.data(), d_part, blocks * sizeof(EvalMoments), hipMemcpyDeviceToHost, stream) == hipSuccess &&
+        ok = hipGetLastError() == hipSuccess && hipMemcpyAsync(mom.data(), d_part, blocks * sizeof(EvalMoments), hipMemcpyDeviceToHost, stream) == hipSuccess &&
              hipStreamSynchronize(stream) == hipSuccess;
     }
     (void)hipFree(d_part);
