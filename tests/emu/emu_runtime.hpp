@@ -332,7 +332,7 @@ thread_local unsigned emu_parity = 0;
 thread_local uint32_t emu_call_seq = 0;
 thread_local bool emu_dirty = false;
 pthread_barrier_t emu_block_barrier;
-emu_alloc emu_allocs[256];
+emu_alloc emu_allocs[1024];
 int emu_n_allocs = 0;
 thread_local hipError_t emu_last_error = hipSuccess;
 pthread_mutex_t emu_alloc_lock = PTHREAD_MUTEX_INITIALIZER, emu_launch_lock = PTHREAD_MUTEX_INITIALIZER;

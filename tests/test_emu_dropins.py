@@ -34,9 +34,9 @@ def test_shim_roundtrip(programs, tmp_path, orc, gen, n):
 
 @pytest.mark.parametrize("variant,ranks,count", [
     ("F", 4, 4 * 32768),               # the reference's own domain: blocks that are multiples of 32768
-    ("F", 3, 100_003),                 # padded blocks, a last block that is mostly padding
+    ("F", 3, 70_003),                  # padded blocks, a last block that is mostly padding
     ("I", 3, 70_000),                  # Lorenzo pre-pass + integer homomorphic sum
-    ("Fseg", 4, 100_003),              # uneven blocks, last block ends with the array
+    ("Fseg", 3, 70_003),               # uneven blocks, last block ends with the array
     ("Iseg", 3, 70_001),
     ("Fseg", 5, 50_000),               # padding pushes the last block's start beyond the array: an empty block
     ("Fopt", 2, 65_536),               # two ranks: no intermediate step

@@ -1,0 +1,139 @@
+"""The gpu-marked parity tests whose sizes the CPU execution model finishes in seconds, run as they
+are (tests/test_gpu_parity.py, the same functions) with the library built for the host
+(libhomcomp_emu.so, tests/emu) behind the same binding and helper: crafted streams of every plane
+count, mode and outlier width, the bit-plane paths, payloads of random bytes under valid headers,
+zero blocks, special values, empty input, truncated sizes, unaligned stream pointers, ragged
+lengths, random mixtures; the plain codec's tests, the tile offsets' and the allocation-free
+entry's argument checks likewise (tests/test_gpu_plain.py, test_gpu_tile_offsets.py,
+test_zz_no_alloc.py)."""
+import importlib.util
+import os
+import sys
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+import test_gpu_parity as parity  # noqa: E402
+import test_gpu_plain as plain  # noqa: E402
+import test_gpu_tile_offsets as tile_offsets  # noqa: E402
+import test_zz_no_alloc as no_alloc  # noqa: E402
+from gpu_util import Gpu  # noqa: E402
+
+
+def _load(name, path):
+    spec = importlib.util.spec_from_file_location(name, path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.fixture(scope="module")
+def emulated():
+    gen_sources = _load("emu_gen_sources", os.path.join(HERE, "emu", "gen_sources.py"))
+    if not os.path.exists(gen_sources.CLANG):
+        pytest.skip("the ROCm clang++ that the host build of the library needs is not installed")
+    harness = _load("emu_harness", os.path.join(HERE, "emu", "harness.py"))
+    os.environ.setdefault("EMU_CUS", "3")
+    return harness.load_binding(gen_sources.build_library()), harness
+
+
+@pytest.fixture()
+def world(emulated):
+    """(the helper on a workspace of the emulated library, the binding, the torch stand-in)"""
+    binding, harness = emulated
+    t = harness.EmuTorch(binding.lib())
+    g = Gpu(binding, t, 1 << 18)
+    yield g, binding, t
+    g.close()
+    t.release()
+
+
+SMALL_CASES = [c for c in parity.CASES if c[1] <= (1 << 16) + 13]
+
+
+@pytest.mark.parametrize("kind,n,mode,val", SMALL_CASES)
+def test_compress_decompress(world, orc, gen, kind, n, mode, val):
+    parity.test_compress_decompress(world[0], orc, gen, kind, n, mode, val)
+
+
+@pytest.mark.parametrize("kind,n,mode,val", [c for c in parity.CASES[:13] if c[1] <= 1 << 17] + SMALL_CASES[:2])
+def test_hom_sums(world, orc, gen, kind, n, mode, val):
+    parity.test_hom_sums(world[0], orc, gen, kind, n, mode, val)
+
+
+def test_every_rate_and_mode(world, orc):
+    parity.test_every_rate_and_mode(world[0], orc)
+
+
+def test_few_planes_per_step(world, orc):
+    parity.test_few_planes_per_step(world[0], orc)
+
+
+def test_sums_in_the_bit_plane_domain(world, orc):
+    parity.test_sums_in_the_bit_plane_domain(world[0], orc)
+
+
+@pytest.mark.parametrize("max_planes", [6, 31])
+def test_arbitrary_payload_bytes(world, orc, max_planes):
+    parity.test_arbitrary_payload_bytes(world[0], orc, max_planes)
+
+
+def test_zero_incoming_blocks(world, orc, gen):
+    parity.test_zero_incoming_blocks(world[0], orc, gen)
+
+
+@pytest.mark.parametrize("special", ["zeros", "constant", "nan_inf", "huge", "alternating"])
+def test_special_values(world, orc, special):
+    parity.test_special_values(world[0], orc, special)
+
+
+def test_empty(world):
+    parity.test_empty(world[0], world[1], world[2])
+
+
+def test_truncated_stream_size(world, orc, gen):
+    parity.test_truncated_stream_size(world[0], orc, gen)
+
+
+@pytest.mark.parametrize("offset", [1, 3, 8, 15])
+def test_unaligned_stream_pointers(world, orc, gen, offset):
+    parity.test_unaligned_stream_pointers(world[0], orc, gen, offset)
+
+
+@pytest.mark.parametrize("seed", [0, 7, 11])
+def test_random_mixtures(world, orc, gen, seed):
+    parity.test_random_mixtures(world[0], orc, gen, seed)
+
+
+def test_argument_errors(world):
+    parity.test_argument_errors(world[0], world[1], world[2])
+
+
+# ---- tests/test_gpu_plain.py
+@pytest.mark.parametrize("kind,n,rel", [c for c in plain.CASES if c[1] <= 1 << 18])
+def test_plain_codec(world, orc, gen, kind, n, rel):
+    plain.test_plain_codec(world[0], orc, gen, kind, n, rel)
+
+
+def test_plain_equals_outlier_codec_without_outlier_blocks(world, orc, gen):
+    plain.test_plain_equals_outlier_codec_without_outlier_blocks(world[0], orc, gen)
+
+
+def test_plain_unaligned_and_saturated(world, orc):
+    plain.test_plain_unaligned_and_saturated(world[0], orc)
+
+
+def test_plain_decoder_reads_no_further_than_the_stream(world, orc, gen):
+    plain.test_plain_decoder_reads_no_further_than_the_stream(world[0], orc, gen)
+
+
+# ---- tests/test_gpu_tile_offsets.py
+@pytest.mark.parametrize("kind,n,rel", [c for c in tile_offsets.CASES if c[1] <= 1 << 18])
+def test_offsets_written_and_taken(world, orc, gen, kind, n, rel):
+    tile_offsets.test_offsets_written_and_taken(world[1], world[2], orc, gen, kind, n, rel)
+
+
+# ---- tests/test_zz_no_alloc.py
+def test_static_entry_limits_and_arguments(world):
+    no_alloc.test_static_entry_limits_and_arguments(world[1], world[2])
