@@ -63,7 +63,7 @@ inline bool emu_device_free(void *p)
 
 // ---------------------------------------------------------------- launches
 // the section of the `__shared__` arrays of this program or library (absent if it has none)
-extern "C" uint8_t __start_emu_lds[] __attribute__((weak)), __stop_emu_lds[] __attribute__((weak));
+extern "C" uint8_t __start_emu_lds[] __attribute__((weak, visibility("hidden"))), __stop_emu_lds[] __attribute__((weak, visibility("hidden")));
 
 // A worker process runs the workgroups first, first + step, ... of a grid one after the other, with
 // one set of lane threads for all of them (starting 256 threads per workgroup is what a large grid

@@ -142,13 +142,21 @@ def build_programs(force: bool = False) -> dict:
     out = os.path.join(GEN, "cpp")
     os.makedirs(out, exist_ok=True)
     paths = {}
-    for name in PROGRAMS:
-        src = os.path.join(os.path.dirname(HERE), "cpp", name + ".cpp")
+    for name in PROGRAMS + ("bitplane_units",):
+        src = os.path.join(os.path.dirname(HERE), "cpp", name + (".hip" if name == "bitplane_units" else ".cpp"))
         exe = paths[name] = os.path.join(out, name)
         deps = [src, library] + [os.path.join(host, f) for f in os.listdir(host)]
         if not force and os.path.exists(exe) and all(os.path.getmtime(f) <= os.path.getmtime(exe) for f in deps):
             continue
-        subprocess.run([CLANG, *CXXFLAGS, "-x", "c++", "-I" + HERE, "-include", os.path.join(HERE, "emu_library_config.h"),
+        if name == "bitplane_units":
+            # the unit program of the bit-plane sums includes the device code itself: the generated one here
+            text = open(src).read()
+            include = '#include "../../tirocinio-triennale_amd/csrc/homcomp_device.hpp"'
+            if text.count(include) != 1:
+                raise SystemExit("gen_sources: bitplane_units.hip includes the device code differently now")
+            src = os.path.join(GEN, "bitplane_units.cpp")
+            open(src, "w").write(text.replace(include, '#include "homcomp_device.hpp"'))
+        subprocess.run([CLANG, *CXXFLAGS, "-x", "c++", "-I" + HERE, "-I" + GEN, "-include", os.path.join(HERE, "emu_library_config.h"),
                         "-o", exe, src, "-L" + GEN, "-lhomcomp_emu", "-Wl,-rpath," + GEN], check=True)
     return paths
 

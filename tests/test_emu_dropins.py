@@ -49,3 +49,12 @@ def test_ring_allreduce(programs, tmp_path, orc, gen, variant, ranks, count):
                                            ("gradient_like", 32768 * 2, 1e-4, 1)])
 def test_evaluator_report(programs, tmp_path, orc, gen, kind, n, eb, rel):
     test_gpu_eval.check_evaluator_report(programs["homcomp_eval"], tmp_path, orc, gen, kind, n, eb, rel, timeout=600)
+
+
+def test_bitplane_sums_against_integer_addition(programs):
+    """tests/cpp/bitplane_units.hip: the sums of the bit-plane paths as device functions alone,
+    against integer addition (here their logic; on the GPU also what the compiler made of them)."""
+    import subprocess
+    res = subprocess.run([programs["bitplane_units"]], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0 and "units ok" in res.stdout, res.stdout + res.stderr
+    assert res.stdout.count(" ok (0 mismatches)") == 9, res.stdout
