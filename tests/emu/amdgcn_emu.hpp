@@ -5,15 +5,19 @@
 // workgroup, device-scope words other workgroups poll).  This header gives those primitives a
 // plain C++ meaning so that the same source text runs on the CPU:
 //
-//   lane        one OS thread; a wave is 64 of them, a workgroup 256 in one process
+//   lane        a fiber (a stack and a saved stack pointer) of its wave's thread; a wave is one
+//               OS thread that runs its 64 lanes in turn, a workgroup four such threads in one
+//               process
 //   workgroup   one process (forked by the driver): `__shared__` becomes `static`, so every
 //               process has its own copy, like every workgroup its own LDS
 //   device      memory: one shared anonymous mapping created before the fork, same addresses in
 //               every process; device-scope atomics are host atomics on it
-//   cross-lane  operations: the lanes of a wave meet at a barrier, exchange through a slot array
-//               and go on (all of them must execute the operation, as on the hardware all lanes
-//               must be active for DPP); wave_lds_fence is a real wave barrier here, because the
-//               lanes do not run in lockstep
+//   cross-lane  operations: the lanes of a wave meet -- each leaves its value and gives way to
+//               the next lane until all that have not left the kernel are there -- exchange
+//               through a slot array and go on.  All of them must be at the same place of the
+//               program, as on the hardware all lanes must be active for DPP: a meeting of
+//               lanes at different places ends the run with a report.  wave_lds_fence is such a
+//               meeting too, because the lanes do not run in lockstep
 //
 // It models what the instruction set defines (lane sources of the DPP controls, byte selectors of
 // v_perm, field extracts, saturating conversion, zero for loads and nothing for stores beyond a
@@ -51,7 +55,6 @@ struct emu_dim3 {
     emu_dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
 };
 typedef emu_dim3 dim3;
-extern thread_local emu_dim3 threadIdx;
 extern emu_dim3 blockIdx, gridDim, blockDim;   // one workgroup per process
 
 // A byte store whose place in the wave's instruction stream matters (see emu_ordered_store8).
@@ -60,16 +63,30 @@ struct emu_store {
     uint32_t seq;
     uint8_t value;
 };
+struct emu_lane_ctx {
+    emu_dim3 tid;        // threadIdx
+    int lane;
+    unsigned parity;     // which of the two slot arrays its next meeting uses
+    uint32_t call_seq;   // see emu_ordered_store8
+    void *sp;            // its stack pointer while another lane runs
+    bool done;           // has left the kernel
+};
 struct emu_wave {
-    pthread_barrier_t bar;
+    emu_lane_ctx lanes[64];
+    unsigned count;            // lanes of the wave (64; fewer in the last wave of an odd workgroup)
+    unsigned live;             // lanes that have not left the kernel
+    unsigned arrived, gen;     // of the meeting under way; meetings so far
+    unsigned site;             // the place in the program the meeting's first lane came from
     uint64_t slot[2][64];
-    uint8_t dirty[2][64];
-    std::vector<emu_store> log[64];
+    std::vector<emu_store> log;
+    void *main_sp;             // the wave thread's own stack pointer while its lanes run
+    const void *kernel;        // std::function<void()> of the launch
 };
 extern thread_local emu_wave *emu_wave_of_thread;
-extern thread_local int emu_lane;
-extern thread_local unsigned emu_parity;
-extern pthread_barrier_t emu_block_barrier;
+extern thread_local emu_lane_ctx *emu_cur;   // the lane that is running on this thread
+#define threadIdx (emu_cur->tid)
+#define emu_lane (emu_cur->lane)
+extern pthread_barrier_t emu_block_barrier;   // of the workgroup's wave threads
 
 // Every access a kernel makes to "device memory" must fall into a registered allocation; the
 // first one that does not is reported with its address and aborts the run.
@@ -97,68 +114,95 @@ inline void emu_check(const void *p, size_t bytes, const char *what)
 // Stores in instruction order.  On the hardware the lanes of a wave execute one instruction
 // together, so of two stores to one address the one later in the program wins, whichever lanes
 // issue them; the encoder's back end relies on that (a lane also writes bytes for planes its
-// block does not have, and a later instruction of another lane overwrites them).  Lanes that are
-// threads have no such order, so these stores are logged with their position in the program
+// block does not have, and a later instruction of another lane overwrites them).  Lanes that run one
+// after the other have no such order, so these stores are logged with their position in the program
 // (`seq`: the count of calls of the storing function so far, which is the same in all lanes, and
 // the store's index inside it) and carried out in that order at the wave's next meeting point.
-extern thread_local uint32_t emu_call_seq;
-extern thread_local bool emu_dirty;
-inline void emu_ordered_enter() { emu_call_seq += 64; }
+inline void emu_ordered_enter() { emu_cur->call_seq += 64; }
 inline void emu_ordered_store8(uint8_t *addr, uint8_t value, uint32_t index)
 {
-    emu_wave_of_thread->log[emu_lane].push_back(emu_store{addr, emu_call_seq + index, value});
-    emu_dirty = true;
+    emu_wave_of_thread->log.push_back(emu_store{addr, emu_cur->call_seq + index, value});
 }
 inline void emu_ordered_store(void *addr, const void *value, uint32_t bytes, uint32_t index)
 {
     for (uint32_t i = 0; i < bytes; ++i) emu_ordered_store8((uint8_t *)addr + i, ((const uint8_t *)value)[i], index);
 }
 inline void emu_ordered_store32(void *addr, uint32_t value, uint32_t index) { emu_ordered_store(addr, &value, 4, index); }
-// after the barrier of a meeting: carries out the logged stores if any lane has some
-inline void emu_flush_stores(emu_wave *w, unsigned p)
+
+// saves the callee-saved registers and the stack pointer of the running lane, takes up another's
+extern "C" void emu_switch(void **save_sp, void *load_sp);
+// gives way to the next lane of the wave that has not left the kernel
+inline void emu_next_lane(emu_wave *w)
 {
-    bool any = false;
-    for (int l = 0; l < 64; ++l) any |= w->dirty[p][l] != 0;
-    if (!any) return;
-    if (emu_lane == 0) {
-        std::vector<emu_store> all;
-        for (int l = 0; l < 64; ++l) {
-            all.insert(all.end(), w->log[l].begin(), w->log[l].end());
-            w->log[l].clear();
-        }
-        std::stable_sort(all.begin(), all.end(), [](const emu_store &a, const emu_store &b) { return a.seq < b.seq; });
-        for (const emu_store &st : all) *st.addr = st.value;
+    emu_lane_ctx *me = emu_cur;
+    unsigned i = (unsigned)me->lane;
+    for (unsigned k = 0; k < w->count; ++k) {
+        i = i + 1 == w->count ? 0 : i + 1;
+        if (!w->lanes[i].done) break;
     }
-    emu_dirty = false;
-    pthread_barrier_wait(&w->bar);
+    emu_lane_ctx *next = &w->lanes[i];
+    if (next == me) {
+        fprintf(stderr, "EMU: lane %d of block %u waits for lanes that have all left the kernel\n", me->lane, blockIdx.x);
+        abort();
+    }
+    emu_cur = next;
+    emu_switch(&me->sp, next->sp);
 }
-// all lanes of the wave meet; each leaves a value and reads another lane's (src < 0: none, gives 0)
-inline uint64_t emu_exchange(uint64_t mine, int src)
+// the last lane to arrive lets the meeting go: the logged stores are carried out in program order first
+inline void emu_release(emu_wave *w)
+{
+    if (!w->log.empty()) {
+        std::stable_sort(w->log.begin(), w->log.end(), [](const emu_store &a, const emu_store &b) { return a.seq < b.seq; });
+        for (const emu_store &st : w->log) *st.addr = st.value;
+        w->log.clear();
+    }
+    w->arrived = 0;
+    w->gen++;
+}
+// All lanes of the wave that have not left the kernel meet; true in the one that arrived last.
+inline bool emu_meet(unsigned site)
 {
     emu_wave *w = emu_wave_of_thread;
-    const unsigned p = emu_parity & 1u;
-    emu_parity++;
+    if (w->arrived == 0) {
+        w->site = site;
+    } else if (w->site != site) {
+        fprintf(stderr, "EMU: the lanes of a wave are at different places of the program (lines %u and %u, lane %d, block %u): "
+                        "a cross-lane operation under a branch that is not uniform\n", w->site, site, emu_cur->lane, blockIdx.x);
+        abort();
+    }
+    const unsigned my = w->gen;
+    if (++w->arrived == w->live) {
+        emu_release(w);
+        return true;
+    }
+    while (w->gen == my) emu_next_lane(w);
+    return false;
+}
+// all lanes meet; each leaves a value and reads another lane's (src < 0: none, gives 0)
+inline uint64_t emu_exchange(unsigned site, uint64_t mine, int src)
+{
+    emu_wave *w = emu_wave_of_thread;
+    const unsigned p = emu_cur->parity++ & 1u;
     w->slot[p][emu_lane] = mine;
-    w->dirty[p][emu_lane] = emu_dirty;
-    pthread_barrier_wait(&w->bar);
-    const uint64_t got = src >= 0 ? w->slot[p][src] : 0;
-    emu_flush_stores(w, p);
-    return got;
+    emu_meet(site);
+    return src >= 0 ? w->slot[p][src] : 0;
 }
 // the same, every lane seeing all values (valid until the lane's next meeting but one)
-inline const uint64_t *emu_gather(uint64_t mine)
+inline const uint64_t *emu_gather(unsigned site, uint64_t mine)
 {
     emu_wave *w = emu_wave_of_thread;
-    const unsigned p = emu_parity & 1u;
-    emu_parity++;
+    const unsigned p = emu_cur->parity++ & 1u;
     w->slot[p][emu_lane] = mine;
-    w->dirty[p][emu_lane] = emu_dirty;
-    pthread_barrier_wait(&w->bar);
-    emu_flush_stores(w, p);
+    emu_meet(site);
     return w->slot[p];
 }
 
-inline void __syncthreads() { pthread_barrier_wait(&emu_block_barrier); }
+// the workgroup's barrier: the lanes of each wave meet, the last one to arrive waits for the other waves
+inline void emu_syncthreads(unsigned site)
+{
+    if (emu_meet(site)) pthread_barrier_wait(&emu_block_barrier);
+}
+#define __syncthreads() emu_syncthreads(__LINE__)
 
 // ---------------------------------------------------------------- cross-lane builtins
 // v_mov_b32 with a DPP control (the controls the kernels use): the lane the value comes from,
@@ -176,38 +220,48 @@ inline int emu_dpp_source(int lane, int ctrl)
     fprintf(stderr, "EMU: DPP control 0x%x is not modelled\n", ctrl);
     abort();
 }
-inline int emu_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl)
+inline int emu_update_dpp(unsigned site, int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl)
 {
     const int lane = emu_lane;
     const int from = emu_dpp_source(lane, ctrl);
-    const uint64_t got = emu_exchange((uint32_t)src, from);
+    const uint64_t got = emu_exchange(site, (uint32_t)src, from);
     const bool enabled = ((row_mask >> (lane >> 4)) & 1) && ((bank_mask >> ((lane >> 2) & 3)) & 1);
     if (!enabled) return old;
     // row_bcast writes only the lanes it has a source for; the others keep `old`
     if (from < 0) return (bound_ctrl && ctrl != 0x142 && ctrl != 0x143) ? 0 : old;
     return (int)(uint32_t)got;
 }
-inline int emu_readfirstlane(int v) { return (int)(uint32_t)emu_exchange((uint32_t)v, 0); }
-inline int emu_readlane(int v, int lane) { return (int)(uint32_t)emu_exchange((uint32_t)v, lane & 63); }
-inline uint64_t emu_ballot(bool pred)
+// (the first lane that is still in the kernel, as the hardware takes the first active one)
+inline int emu_readfirstlane(unsigned site, int v)
 {
-    const uint64_t *all = emu_gather(pred ? 1u : 0u);
+    const emu_wave *w = emu_wave_of_thread;
+    int first = 0;
+    while (first < 63 && w->lanes[first].done) ++first;
+    return (int)(uint32_t)emu_exchange(site, (uint32_t)v, first);
+}
+inline int emu_readlane(unsigned site, int v, int lane) { return (int)(uint32_t)emu_exchange(site, (uint32_t)v, lane & 63); }
+inline uint64_t emu_ballot(unsigned site, bool pred)
+{
+    const uint64_t *all = emu_gather(site, pred ? 1u : 0u);
+    const emu_wave *w = emu_wave_of_thread;
     uint64_t m = 0;
-    for (int l = 0; l < 64; ++l) m |= (all[l] & 1u) << l;
+    for (unsigned l = 0; l < w->count; ++l)
+        if (!w->lanes[l].done) m |= (all[l] & 1u) << l;
     return m;
 }
 template <typename T>
-inline T __shfl_xor(T v, int mask, int /*width*/)
+inline T emu_shfl_xor(unsigned site, T v, int mask, int /*width*/)
 {
     static_assert(sizeof(T) <= 8, "values of up to 64 bits");
     uint64_t bits = 0;
     memcpy(&bits, &v, sizeof(T));
-    const uint64_t got = emu_exchange(bits, (emu_lane ^ mask) & 63);
+    const uint64_t got = emu_exchange(site, bits, (emu_lane ^ mask) & 63);
     T out;
     memcpy(&out, &got, sizeof(T));
     return out;
 }
-inline void emu_wave_barrier() { (void)emu_exchange(0, -1); }
+#define __shfl_xor(v, mask, width) emu_shfl_xor(__LINE__, v, mask, width)
+inline void emu_wave_barrier(unsigned site) { (void)emu_meet(site); }
 
 // ---------------------------------------------------------------- lane-local builtins
 inline uint32_t emu_perm(uint32_t s0, uint32_t s1, uint32_t sel)
@@ -273,20 +327,31 @@ struct emu_rsrc {
 typedef unsigned int emu_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int emu_u32x2 __attribute__((ext_vector_type(2)));
 inline emu_rsrc emu_make_rsrc(void *base, short /*stride*/, int bytes, int /*flags*/) { return emu_rsrc{(uint8_t *)base, (uint32_t)bytes}; }
-// dword d of an access at `off` is in range when it ends within the descriptor's byte count
+// dword d of an access at `off` is in range when it ends within the descriptor's byte count.
+// An aligned pair of dwords is moved as one 64-bit access, a dword as one 32-bit access: the
+// hardware does not tear them, and the status words other workgroups poll rely on that.
 template <int DWORDS>
 inline void emu_buf_load(const emu_rsrc &rs, uint32_t voff, uint32_t soff, uint32_t *out)
 {
     const uint64_t off = (uint64_t)voff + soff;
     for (int d = 0; d < DWORDS; ++d) {
         out[d] = 0;
-        if (off + 4u * d + 4u <= rs.bytes) {
-            emu_check(rs.base + off + 4u * d, 4, "buffer load");
-            memcpy(&out[d], rs.base + off + 4u * d, 4);
+        const uint8_t *at = rs.base + off + 4u * d;
+        if (d + 1 < DWORDS && ((uintptr_t)at & 7u) == 0 && off + 4u * d + 8u <= rs.bytes) {
+            emu_check(at, 8, "buffer load");
+            const uint64_t v = __atomic_load_n((const uint64_t *)at, __ATOMIC_SEQ_CST);
+            out[d] = (uint32_t)v;
+            out[++d] = (uint32_t)(v >> 32);
+        } else if (off + 4u * d + 4u <= rs.bytes) {
+            emu_check(at, 4, "buffer load");
+            if (((uintptr_t)at & 3u) == 0)
+                out[d] = __atomic_load_n((const uint32_t *)at, __ATOMIC_SEQ_CST);
+            else
+                memcpy(&out[d], at, 4);
         } else if (off + 4u * d < rs.bytes) {   // a dword that straddles the end: the bytes below it
             const uint32_t n = (uint32_t)(rs.bytes - (off + 4u * d));
-            emu_check(rs.base + off + 4u * d, n, "buffer load");
-            memcpy(&out[d], rs.base + off + 4u * d, n);
+            emu_check(at, n, "buffer load");
+            memcpy(&out[d], at, n);
         }
     }
 }
@@ -294,11 +359,20 @@ template <int DWORDS>
 inline void emu_buf_store(const emu_rsrc &rs, uint32_t voff, uint32_t soff, const uint32_t *in)
 {
     const uint64_t off = (uint64_t)voff + soff;
-    for (int d = 0; d < DWORDS; ++d)
-        if (off + 4u * d + 4u <= rs.bytes) {
-            emu_check(rs.base + off + 4u * d, 4, "buffer store");
-            memcpy(rs.base + off + 4u * d, &in[d], 4);
+    for (int d = 0; d < DWORDS; ++d) {
+        uint8_t *at = rs.base + off + 4u * d;
+        if (d + 1 < DWORDS && ((uintptr_t)at & 7u) == 0 && off + 4u * d + 8u <= rs.bytes) {
+            emu_check(at, 8, "buffer store");
+            __atomic_store_n((uint64_t *)at, (uint64_t)in[d] | ((uint64_t)in[d + 1] << 32), __ATOMIC_SEQ_CST);
+            ++d;
+        } else if (off + 4u * d + 4u <= rs.bytes) {
+            emu_check(at, 4, "buffer store");
+            if (((uintptr_t)at & 3u) == 0)
+                __atomic_store_n((uint32_t *)at, in[d], __ATOMIC_SEQ_CST);
+            else
+                memcpy(at, &in[d], 4);
         }
+    }
 }
 inline emu_u32x4 emu_load_b128(emu_rsrc rs, int voff, int soff, int)
 {
@@ -356,28 +430,32 @@ inline void emu_store_b8(uint8_t v, emu_rsrc rs, int voff, int soff, int)
 #define __builtin_amdgcn_raw_buffer_store_b128 emu_store_b128
 #define __builtin_amdgcn_raw_buffer_store_b64 emu_store_b64
 #define __builtin_amdgcn_raw_buffer_store_b8 emu_store_b8
-#define __builtin_amdgcn_update_dpp emu_update_dpp
-#define __builtin_amdgcn_readfirstlane emu_readfirstlane
-#define __builtin_amdgcn_readlane emu_readlane
-#define __builtin_amdgcn_ballot_w64 emu_ballot
+#define __builtin_amdgcn_update_dpp(...) emu_update_dpp(__LINE__, __VA_ARGS__)
+#define __builtin_amdgcn_readfirstlane(...) emu_readfirstlane(__LINE__, __VA_ARGS__)
+#define __builtin_amdgcn_readlane(...) emu_readlane(__LINE__, __VA_ARGS__)
+#define __builtin_amdgcn_ballot_w64(...) emu_ballot(__LINE__, __VA_ARGS__)
 #define __builtin_amdgcn_perm emu_perm
 #define __builtin_amdgcn_alignbit emu_alignbit
 #define __builtin_amdgcn_alignbyte emu_alignbyte
 #define __builtin_amdgcn_ubfe emu_ubfe
 #define __builtin_amdgcn_sbfe emu_sbfe
 #define __builtin_amdgcn_sad_u8 emu_sad_u8
-// A wave that sleeps between two looks at a word another workgroup writes: the bounds on such waits
-// count looks, and are sized for a device on which every workgroup runs at once; here a
-// workgroup may have to wait for a processor, so a look takes its time
+// A lane that sleeps between two looks at a word another workgroup writes.  On the hardware the
+// other lanes of its wave go on meanwhile; here they run on the same thread, so the lane gives
+// way to them first (what it waits for may depend on a store one of them has not made yet), then
+// the thread sleeps: the bounds on such waits count looks and are sized for a device on which
+// every workgroup runs at once, while here a workgroup may have to wait for a processor.
 inline void emu_sleep()
 {
-    const timespec t{0, 20000};
+    emu_wave *w = emu_wave_of_thread;
+    if (w && w->live > 1) emu_next_lane(w);
+    const timespec t{0, 100000};
     nanosleep(&t, nullptr);
 }
 #define __builtin_amdgcn_s_sleep(n) emu_sleep()
 #define __builtin_amdgcn_s_setprio(n) ((void)0)
 #define __builtin_amdgcn_fence(order, scope) __atomic_thread_fence(__ATOMIC_SEQ_CST)
-#define __builtin_amdgcn_wave_barrier emu_wave_barrier
+#define __builtin_amdgcn_wave_barrier() emu_wave_barrier(__LINE__)
 
 // device-scope atomics: host atomics on the shared mapping
 #define __HIP_MEMORY_SCOPE_AGENT 0

@@ -66,60 +66,99 @@ inline bool emu_device_free(void *p)
 extern "C" uint8_t __start_emu_lds[] __attribute__((weak, visibility("hidden"))), __stop_emu_lds[] __attribute__((weak, visibility("hidden")));
 
 // A worker process runs the workgroups first, first + step, ... of a grid one after the other, with
-// one set of lane threads for all of them (starting 256 threads per workgroup is what a large grid
-// of small workgroups would otherwise spend its time on).
+// one thread per wave and one set of lane stacks for all of them.
 struct emu_worker {
     const std::function<void()> *kernel;
-    emu_wave *waves;
     unsigned threads, first, step, blocks, grid_x;
 };
-struct emu_lane_start {
+struct emu_wave_start {
     const emu_worker *worker;
-    int tid;
+    unsigned index;   // of the wave in its workgroup
 };
-inline void *emu_lane_main(void *arg)
+const size_t emu_lane_stack = 1 << 20;   // per lane; only the pages a lane touches exist
+
+// where a lane starts, and where it ends up when it leaves the kernel
+extern "C" inline void emu_lane_entry()
 {
-    const emu_lane_start *s = (const emu_lane_start *)arg;
-    const emu_worker *w = s->worker;
-    threadIdx.x = (unsigned)s->tid;
-    emu_lane = s->tid & 63;
-    emu_wave_of_thread = &w->waves[s->tid / 64];
-    for (unsigned i = w->first; i < w->blocks; i += w->step) {
-        if (s->tid == 0) {
-            blockIdx.x = i % w->grid_x;
-            blockIdx.y = i / w->grid_x;
+    emu_wave *w = emu_wave_of_thread;
+    (*(const std::function<void()> *)w->kernel)();
+    emu_lane_ctx *me = emu_cur;
+    me->done = true;
+    w->live--;
+    if (w->live == 0) {
+        emu_switch(&me->sp, w->main_sp);   // the wave is through; does not come back
+    }
+    if (w->arrived == w->live) emu_release(w);   // the others were waiting for this lane only
+    emu_next_lane(w);                             // does not come back either
+    abort();
+}
+
+inline void *emu_wave_main(void *arg)
+{
+    const emu_wave_start *s = (const emu_wave_start *)arg;
+    const emu_worker *k = s->worker;
+    emu_wave *w = new emu_wave;
+    emu_wave_of_thread = w;
+    w->kernel = k->kernel;
+    w->count = k->threads - 64 * s->index < 64 ? k->threads - 64 * s->index : 64;
+    uint8_t *stacks = (uint8_t *)mmap(nullptr, 64 * emu_lane_stack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (stacks == MAP_FAILED) {
+        perror("EMU: lane stacks");
+        _exit(3);
+    }
+    for (unsigned l = 0; l < 64; ++l) mprotect(stacks + l * emu_lane_stack, emu_page, PROT_NONE);   // a lane that outgrows its stack faults
+    for (unsigned i = k->first; i < k->blocks; i += k->step) {
+        if (s->index == 0) {
+            blockIdx.x = i % k->grid_x;
+            blockIdx.y = i / k->grid_x;
             // LDS as the workgroup finds it: not zeros
             for (uint8_t *b = __start_emu_lds; b && b != __stop_emu_lds; ++b) *b = (uint8_t)(0xC3u ^ (uintptr_t)b * 37u ^ i * 11u);
         }
-        emu_parity = 0;
-        emu_call_seq = 0;
-        emu_dirty = false;
+        for (unsigned l = 0; l < w->count; ++l) {
+            emu_lane_ctx &c = w->lanes[l];
+            c.tid = emu_dim3(64 * s->index + l);
+            c.lane = (int)l;
+            c.parity = 0;
+            c.call_seq = 0;
+            c.done = false;
+            // the frame emu_switch pops: six callee-saved registers, then the address it returns to; the
+            // stack pointer after that return is 8 below a multiple of 16, as at any function's entry
+            uint64_t *top = (uint64_t *)(stacks + (l + 1) * emu_lane_stack);
+            top[-2] = (uint64_t)(uintptr_t)&emu_lane_entry;
+            for (int r = 3; r <= 8; ++r) top[-r] = 0;
+            c.sp = top - 8;
+        }
+        w->live = w->count;
+        w->arrived = 0;
+        w->gen = 0;
+        w->log.clear();
         pthread_barrier_wait(&emu_block_barrier);
-        (*w->kernel)();
+        emu_cur = &w->lanes[0];
+        emu_switch(&w->main_sp, w->lanes[0].sp);   // back here when the wave's last lane has left the kernel
         pthread_barrier_wait(&emu_block_barrier);
     }
+    munmap(stacks, 64 * emu_lane_stack);
+    delete w;
     return nullptr;
 }
 
-inline void emu_run_worker(emu_worker &w)
+inline void emu_run_worker(emu_worker &k)
 {
-    const unsigned threads = w.threads, waves = (threads + 63) / 64;
-    w.waves = new emu_wave[waves];
-    for (unsigned i = 0; i < waves; ++i) pthread_barrier_init(&w.waves[i].bar, nullptr, i + 1 < waves || threads % 64 == 0 ? 64 : threads % 64);
-    pthread_barrier_init(&emu_block_barrier, nullptr, threads);
-    pthread_t *th = new pthread_t[threads];
-    emu_lane_start *st = new emu_lane_start[threads];
+    const unsigned waves = (k.threads + 63) / 64;
+    pthread_barrier_init(&emu_block_barrier, nullptr, waves);
+    pthread_t *th = new pthread_t[waves];
+    emu_wave_start *st = new emu_wave_start[waves];
     pthread_attr_t attr;
     pthread_attr_init(&attr);
     pthread_attr_setstacksize(&attr, 1 << 20);
-    for (unsigned t = 0; t < threads; ++t) {
-        st[t] = emu_lane_start{&w, (int)t};
-        if (pthread_create(&th[t], &attr, emu_lane_main, &st[t]) != 0) {
+    for (unsigned i = 0; i < waves; ++i) {
+        st[i] = emu_wave_start{&k, i};
+        if (pthread_create(&th[i], &attr, emu_wave_main, &st[i]) != 0) {
             perror("EMU: pthread_create");
             _exit(3);
         }
     }
-    for (unsigned t = 0; t < threads; ++t) pthread_join(th[t], nullptr);
+    for (unsigned i = 0; i < waves; ++i) pthread_join(th[i], nullptr);
 }
 
 // A grid.  Up to emu_resident_limit() workgroups are alive at the same time, each in a process of
@@ -153,7 +192,7 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
             break;
         }
         if (k == 0) {
-            emu_worker w{&kernel, nullptr, block.x, i, workers, n, grid.x};
+            emu_worker w{&kernel, block.x, i, workers, n, grid.x};
             emu_run_worker(w);
             fflush(nullptr);
             _exit(0);
@@ -324,16 +363,36 @@ inline hipError_t hipGetSymbolAddress(void **p, const void *symbol, size_t bytes
 }
 
 #ifdef EMU_DEFINE_GLOBALS
-thread_local emu_dim3 threadIdx;
 emu_dim3 blockIdx, gridDim, blockDim;
 thread_local emu_wave *emu_wave_of_thread = nullptr;
-thread_local int emu_lane = 0;
-thread_local unsigned emu_parity = 0;
-thread_local uint32_t emu_call_seq = 0;
-thread_local bool emu_dirty = false;
+thread_local emu_lane_ctx *emu_cur = nullptr;
 pthread_barrier_t emu_block_barrier;
 emu_alloc emu_allocs[1024];
 int emu_n_allocs = 0;
 thread_local hipError_t emu_last_error = hipSuccess;
 pthread_mutex_t emu_alloc_lock = PTHREAD_MUTEX_INITIALIZER, emu_launch_lock = PTHREAD_MUTEX_INITIALIZER;
+// emu_switch(save_sp, load_sp), x86-64 System V: the registers a call preserves go onto the running
+// lane's stack, its stack pointer into *save_sp; the other lane's are taken up the same way round
+asm(R"(
+    .text
+    .globl emu_switch
+    .type emu_switch,@function
+emu_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+    .size emu_switch, .-emu_switch
+)");
 #endif

@@ -42,7 +42,7 @@ KERNEL_EDITS = [
     # A wave's LDS instructions take effect in the order of the program, for all its lanes: what the lanes packed is
     # in the stage when the instructions that move it elsewhere read it.  Lanes that are threads have to meet for that.
     ("            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {\n",
-     "            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {\n                emu_wave_barrier();\n"),
+     "            auto make_room = [&](uint32_t bytes) __attribute__((always_inline)) {\n                emu_wave_barrier(__LINE__);\n"),
 ]
 LAUNCHERS = "// ---------------------------------------------------------------- launchers"
 

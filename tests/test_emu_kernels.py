@@ -1,4 +1,4 @@
-"""The kernels' source text executed on the CPU (tests/emu: lanes as threads, workgroups as
+"""The kernels' source text executed on the CPU (tests/emu: lanes as fibers of their wave's thread, workgroups as
 processes, device memory as guarded shared mappings) against the oracle, byte for byte, on small
 inputs.  It covers what a GPU run covers less directly: every path of every kernel kind on data
 that does and does not suit it, whatever the launch heuristics would pick; grids of one and of
