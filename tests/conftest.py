@@ -25,17 +25,69 @@ def orc():
 
 @pytest.fixture(scope="session")
 def gen():
-    return entry.load_datagen()
+    datagen = entry.load_datagen()
+    model = _cpu_model()
+    if not model:
+        return datagen
+
+    class OnTheModel:
+        """The generators; the ones that produce device tensors go through their numpy twins
+        (the same values) into the model's device memory."""
+        GENERATORS_TORCH = {kind: (lambda n, seed=1, _f=f: model["torch"].from_numpy(_f(n, seed)).cuda())
+                            for kind, f in datagen.GENERATORS_NP.items()}
+
+        def __getattr__(self, name):
+            return getattr(datagen, name)
+    return OnTheModel()
+
+
+def _cpu_model():
+    """HOMCOMP_CPU_MODEL=1 points the gpu-marked tests at the library built for the host against
+    the CPU execution model (tests/emu) instead of the GPU: the same binding bound to
+    libhomcomp_emu.so and a stand-in for the torch calls the tests make.  For looking at a test's
+    logic without a GPU (the ones whose sizes the model can finish; graphs, side-by-side streams
+    and memory queries do not exist there); what counts as GPU parity is a run without it."""
+    if os.environ.get("HOMCOMP_CPU_MODEL", "0") in ("", "0"):
+        return None
+    if "binding" not in _model:
+        import importlib.util
+
+        def load(name, path):
+            spec = importlib.util.spec_from_file_location(name, path)
+            mod = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(mod)
+            return mod
+        here = os.path.join(ROOT, "tests", "emu")
+        harness = load("emu_harness", os.path.join(here, "harness.py"))
+        os.environ.setdefault("EMU_CUS", "5")
+        _model["binding"] = harness.load_binding(load("emu_gen_sources", os.path.join(here, "gen_sources.py")).build_library())
+        _model["torch"] = harness.EmuTorch(_model["binding"].lib())
+    return _model
+
+
+_model = {}
+
+
+@pytest.fixture(autouse=True)
+def _release_model_buffers():
+    """(CPU model only) the buffers a test allocated through the torch stand-in go back when it ends."""
+    yield
+    if "torch" in _model:
+        _model["torch"].release()
 
 
 @pytest.fixture(scope="session")
 def pkg():
     """The product package; loading it fails loudly when libhomcomp_amd.so is missing."""
-    return entry.load_package()
+    model = _cpu_model()
+    return model["binding"] if model else entry.load_package()
 
 
 @pytest.fixture(scope="session")
 def cuda():
+    model = _cpu_model()
+    if model:
+        return model["torch"]
     import torch
     if not torch.cuda.is_available():
         pytest.fail("GPU test selected but no GPU is available")

@@ -96,7 +96,7 @@ struct emu_alloc {
     uintptr_t map;      // the mapping around it (guard pages included), for its release
     size_t map_bytes;
 };
-extern emu_alloc emu_allocs[1024];
+extern emu_alloc emu_allocs[8192];
 extern int emu_n_allocs;
 inline void emu_check(const void *p, size_t bytes, const char *what)
 {

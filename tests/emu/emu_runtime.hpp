@@ -295,7 +295,7 @@ inline int emu_compute_units()
 {
     const char *e = getenv("EMU_CUS");
     const int v = e ? atoi(e) : 3;
-    return v < 1 ? 1 : (v > 16 ? 16 : v);
+    return v < 1 ? 1 : (v > 256 ? 256 : v);
 }
 inline hipError_t hipGetDeviceProperties(hipDeviceProp_t *prop, int)
 {
@@ -367,7 +367,7 @@ emu_dim3 blockIdx, gridDim, blockDim;
 thread_local emu_wave *emu_wave_of_thread = nullptr;
 thread_local emu_lane_ctx *emu_cur = nullptr;
 pthread_barrier_t emu_block_barrier;
-emu_alloc emu_allocs[1024];
+emu_alloc emu_allocs[8192];
 int emu_n_allocs = 0;
 thread_local hipError_t emu_last_error = hipSuccess;
 pthread_mutex_t emu_alloc_lock = PTHREAD_MUTEX_INITIALIZER, emu_launch_lock = PTHREAD_MUTEX_INITIALIZER;
