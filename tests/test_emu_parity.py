@@ -1,5 +1,5 @@
-"""The gpu-marked parity tests whose sizes the CPU execution model finishes in seconds, run as they
-are (tests/test_gpu_parity.py, the same functions) with the library built for the host
+"""The gpu-marked parity tests, all but the three that need graphs or streams side by side, run as
+they are (tests/test_gpu_parity.py, the same functions) with the library built for the host
 (libhomcomp_emu.so, tests/emu) behind the same binding and helper: crafted streams of every plane
 count, mode and outlier width, the bit-plane paths, payloads of random bytes under valid headers,
 zero blocks, special values, empty input, truncated sizes, unaligned stream pointers, ragged
@@ -43,21 +43,18 @@ def world(emulated):
     """(the helper on a workspace of the emulated library, the binding, the torch stand-in)"""
     binding, harness = emulated
     t = harness.EmuTorch(binding.lib())
-    g = Gpu(binding, t, 1 << 18)
+    g = Gpu(binding, t, parity.MAX_N)
     yield g, binding, t
     g.close()
     t.release()
 
 
-SMALL_CASES = [c for c in parity.CASES if c[1] <= (1 << 16) + 13]
-
-
-@pytest.mark.parametrize("kind,n,mode,val", SMALL_CASES)
+@pytest.mark.parametrize("kind,n,mode,val", parity.CASES)
 def test_compress_decompress(world, orc, gen, kind, n, mode, val):
     parity.test_compress_decompress(world[0], orc, gen, kind, n, mode, val)
 
 
-@pytest.mark.parametrize("kind,n,mode,val", [c for c in parity.CASES[:13] if c[1] <= 1 << 17] + SMALL_CASES[:2])
+@pytest.mark.parametrize("kind,n,mode,val", parity.CASES[:13])
 def test_hom_sums(world, orc, gen, kind, n, mode, val):
     parity.test_hom_sums(world[0], orc, gen, kind, n, mode, val)
 
@@ -96,18 +93,55 @@ def test_truncated_stream_size(world, orc, gen):
     parity.test_truncated_stream_size(world[0], orc, gen)
 
 
-@pytest.mark.parametrize("offset", [1, 3, 8, 15])
+@pytest.mark.parametrize("offset", [1, 2, 3, 5, 8, 15])
 def test_unaligned_stream_pointers(world, orc, gen, offset):
     parity.test_unaligned_stream_pointers(world[0], orc, gen, offset)
 
 
-@pytest.mark.parametrize("seed", [0, 7, 11])
+@pytest.mark.parametrize("seed", range(12))
 def test_random_mixtures(world, orc, gen, seed):
     parity.test_random_mixtures(world[0], orc, gen, seed)
 
 
 def test_argument_errors(world):
     parity.test_argument_errors(world[0], world[1], world[2])
+
+
+def test_value_range(world, orc, gen):
+    parity.test_value_range(world[0], orc, gen, world[1])
+
+
+def test_workspace_reuse_many_calls(world, orc, gen):
+    parity.test_workspace_reuse_many_calls(world[0], orc, gen)
+
+
+@pytest.mark.parametrize("grid_percent", [1])
+def test_many_rounds_and_small_grids(world, orc, gen, monkeypatch, grid_percent):
+    parity.test_many_rounds_and_small_grids(world[1], world[2], orc, gen, monkeypatch, grid_percent)
+
+
+@pytest.mark.parametrize("stage,slots", [("small", 4)])
+def test_lds_budgets_and_deferral_depths(world, orc, gen, monkeypatch, stage, slots):
+    parity.test_lds_budgets_and_deferral_depths(world[1], world[2], orc, gen, monkeypatch, stage, slots)
+
+
+def test_lds_budget_follows_the_data(world, orc, gen):
+    parity.test_lds_budget_follows_the_data(world[1], world[2], orc, gen)
+
+
+@pytest.mark.parametrize("forced", [None, "2"])
+def test_sum_kernel_follows_the_incoming_tiles(world, orc, gen, monkeypatch, forced):
+    parity.test_sum_kernel_follows_the_incoming_tiles(world[1], world[2], orc, gen, monkeypatch, forced)
+
+
+@pytest.mark.parametrize("forced", [None, "2", "3"])
+def test_stream_plus_stream_wide_blocks(world, orc, monkeypatch, forced):
+    parity.test_stream_plus_stream_wide_blocks(world[1], world[2], orc, monkeypatch, forced)
+
+
+@pytest.mark.parametrize("tiles,offset", [(2049, 5)])
+def test_offsets_prepass_sizes(world, orc, gen, tiles, offset):
+    parity.test_offsets_prepass_sizes(world[1], world[2], orc, gen, tiles, offset)
 
 
 # ---- tests/test_gpu_plain.py
