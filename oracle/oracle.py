@@ -161,19 +161,42 @@ def block_decode(hdr: int, payload: bytes) -> np.ndarray:
     return d
 
 
+_CANARY = 64   # bytes behind every output array that the C side must leave alone
+
+
+def _out(count: int, dtype) -> np.ndarray:
+    """A zeroed output array of `count` elements with a canary behind it (see _done)."""
+    item = np.dtype(dtype).itemsize
+    raw = np.zeros(count * item + _CANARY, np.uint8)
+    raw[count * item:] = 0x5C
+    return raw
+
+
+def _view(raw: np.ndarray, count: int, dtype) -> np.ndarray:
+    return raw[:count * np.dtype(dtype).itemsize].view(dtype)
+
+
+def _done(raw: np.ndarray, count: int, dtype) -> np.ndarray:
+    """The output proper, after checking that nothing was written behind it."""
+    item = np.dtype(dtype).itemsize
+    assert (raw[count * item:] == 0x5C).all(), "the oracle wrote beyond its output array"
+    return raw[:count * item].view(dtype)
+
+
 def quantize_array(x, eb: float) -> np.ndarray:
     x = _f32(x)
-    q = np.empty(x.size, np.int32)
+    q = _out(x.size, np.int32)
     lib().hco_quantize_array(_p(x, C.c_float), x.size, np.float32(eb), _p(q, C.c_int32))
-    return q
+    return _done(q, x.size, np.int32)
 
 
 def quant_predict(x, eb: float, padded: bool = False) -> np.ndarray:
     x = _f32(x)
     n = x.size
-    d = np.empty(padded_len(n) if padded else n, np.int32)
+    count = padded_len(n) if padded else n
+    d = _out(count, np.int32)
     lib().hco_quant_predict(_p(x, C.c_float), n, np.float32(eb), _p(d, C.c_int32), int(padded))
-    return d
+    return _done(d, count, np.int32)
 
 
 def compress(x, eb: float, want_offsets: bool = False):
@@ -181,33 +204,35 @@ def compress(x, eb: float, want_offsets: bool = False):
     absolute payload offset of every block (padded_blocks + 1 entries)."""
     x = _f32(x)
     n = x.size
-    cmp = np.zeros(max_stream_bytes(n), np.uint8)
+    cap = max_stream_bytes(n)
+    cmp = _out(cap, np.uint8)
     L = C.c_size_t()
-    ofs = np.zeros(header_bytes(n) + 1, np.uint64) if want_offsets else None
+    ofs = _out(header_bytes(n) + 1, np.uint64) if want_offsets else None
     rc = lib().hco_compress(_p(x, C.c_float), n, np.float32(eb), _p(cmp, C.c_uint8), C.byref(L),
                             _p(ofs, C.c_uint64) if want_offsets else None)
-    assert rc == 0
-    out = cmp[:L.value].copy()
-    return (out, ofs) if want_offsets else out
+    assert rc == 0 and L.value <= cap
+    out = _done(cmp, cap, np.uint8)[:L.value].copy()
+    return (out, _done(ofs, header_bytes(n) + 1, np.uint64)) if want_offsets else out
 
 
 def compress_plain(x, eb: float) -> np.ndarray:
     """The plain codec's stream (true length)."""
     x = _f32(x)
     n = x.size
-    cmp = np.zeros(max_stream_bytes(n) + 4 * header_bytes(n), np.uint8)
+    cap = max_stream_bytes(n) + 4 * header_bytes(n)
+    cmp = _out(cap, np.uint8)
     L = C.c_size_t()
     rc = lib().hco_compress_plain(_p(x, C.c_float), n, np.float32(eb), _p(cmp, C.c_uint8), C.byref(L))
-    assert rc == 0
-    return cmp[:L.value].copy()
+    assert rc == 0 and L.value <= cap
+    return _done(cmp, cap, np.uint8)[:L.value].copy()
 
 
 def decompress_plain(cmp, n: int, eb: float) -> np.ndarray:
     buf = _padded_stream(cmp, n)
-    out = np.zeros(n, np.float32)
+    out = _out(n, np.float32)
     rc = lib().hco_decompress_plain(_p(buf, C.c_uint8), n, np.float32(eb), _p(out, C.c_float))
     assert rc == 0
-    return out
+    return _done(out, n, np.float32)
 
 
 def block_encode_plain(delta) -> tuple[int, bytes]:
@@ -222,11 +247,12 @@ def block_encode_plain(delta) -> tuple[int, bytes]:
 def encode_deltas(delta) -> np.ndarray:
     d = _i32(delta)
     n = d.size
-    cmp = np.zeros(max_stream_bytes(n), np.uint8)
+    cap = max_stream_bytes(n)
+    cmp = _out(cap, np.uint8)
     L = C.c_size_t()
     rc = lib().hco_encode_deltas(_p(d, C.c_int32), n, _p(cmp, C.c_uint8), C.byref(L))
-    assert rc == 0
-    return cmp[:L.value].copy()
+    assert rc == 0 and L.value <= cap
+    return _done(cmp, cap, np.uint8)[:L.value].copy()
 
 
 def _padded_stream(cmp, n: int) -> np.ndarray:
@@ -242,30 +268,30 @@ def decompress(cmp, n: int, eb: float, cmp_size: int | None = None) -> np.ndarra
     cmp = _u8(cmp)
     size = cmp.size if cmp_size is None else cmp_size
     buf = _padded_stream(cmp, n)
-    out = np.zeros(n, np.float32)
+    out = _out(n, np.float32)
     rc = lib().hco_decompress(_p(buf, C.c_uint8), size, n, np.float32(eb), _p(out, C.c_float))
     assert rc == 0
-    return out
+    return _done(out, n, np.float32)
 
 
 def decode_deltas(cmp, n: int, cmp_size: int | None = None) -> np.ndarray:
     cmp = _u8(cmp)
     size = cmp.size if cmp_size is None else cmp_size
     buf = _padded_stream(cmp, n)
-    out = np.zeros(n, np.int32)
+    out = _out(n, np.int32)
     rc = lib().hco_decode_deltas(_p(buf, C.c_uint8), size, n, _p(out, C.c_int32))
     assert rc == 0
-    return out
+    return _done(out, n, np.int32)
 
 
 def decode_quants(cmp, n: int, cmp_size: int | None = None) -> np.ndarray:
     cmp = _u8(cmp)
     size = cmp.size if cmp_size is None else cmp_size
     buf = _padded_stream(cmp, n)
-    out = np.zeros(n, np.int32)
+    out = _out(n, np.int32)
     rc = lib().hco_decode_quants(_p(buf, C.c_uint8), size, n, _p(out, C.c_int32))
     assert rc == 0
-    return out
+    return _done(out, n, np.int32)
 
 
 def hom_sum_f32(cmp_in, local, eb: float, cmp_in_size: int | None = None) -> np.ndarray:
@@ -274,12 +300,13 @@ def hom_sum_f32(cmp_in, local, eb: float, cmp_in_size: int | None = None) -> np.
     cmp_in = _u8(cmp_in)
     size = cmp_in.size if cmp_in_size is None else cmp_in_size
     buf = _padded_stream(cmp_in, n)
-    out = np.zeros(max_stream_bytes(n), np.uint8)
+    cap = max_stream_bytes(n)
+    out = _out(cap, np.uint8)
     L = C.c_size_t()
     rc = lib().hco_hom_sum_f32(_p(buf, C.c_uint8), size, _p(local, C.c_float), n,
                                np.float32(eb), _p(out, C.c_uint8), C.byref(L))
-    assert rc == 0
-    return out[:L.value].copy()
+    assert rc == 0 and L.value <= cap
+    return _done(out, cap, np.uint8)[:L.value].copy()
 
 
 def hom_sum_i32(cmp_in, local_delta, cmp_in_size: int | None = None) -> np.ndarray:
@@ -288,21 +315,23 @@ def hom_sum_i32(cmp_in, local_delta, cmp_in_size: int | None = None) -> np.ndarr
     cmp_in = _u8(cmp_in)
     size = cmp_in.size if cmp_in_size is None else cmp_in_size
     buf = _padded_stream(cmp_in, n)
-    out = np.zeros(max_stream_bytes(n), np.uint8)
+    cap = max_stream_bytes(n)
+    out = _out(cap, np.uint8)
     L = C.c_size_t()
     rc = lib().hco_hom_sum_i32(_p(buf, C.c_uint8), size, _p(d, C.c_int32), n,
                                _p(out, C.c_uint8), C.byref(L))
-    assert rc == 0
-    return out[:L.value].copy()
+    assert rc == 0 and L.value <= cap
+    return _done(out, cap, np.uint8)[:L.value].copy()
 
 
 def hom_add(cmp_a, cmp_b, n: int, size_a: int | None = None, size_b: int | None = None) -> np.ndarray:
     a, b = _u8(cmp_a), _u8(cmp_b)
     ba, bb = _padded_stream(a, n), _padded_stream(b, n)
-    out = np.zeros(max_stream_bytes(n), np.uint8)
+    cap = max_stream_bytes(n)
+    out = _out(cap, np.uint8)
     L = C.c_size_t()
     rc = lib().hco_hom_add(_p(ba, C.c_uint8), a.size if size_a is None else size_a,
                            _p(bb, C.c_uint8), b.size if size_b is None else size_b, n,
                            _p(out, C.c_uint8), C.byref(L))
-    assert rc == 0
-    return out[:L.value].copy()
+    assert rc == 0 and L.value <= cap
+    return _done(out, cap, np.uint8)[:L.value].copy()

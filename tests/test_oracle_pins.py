@@ -46,6 +46,11 @@ def test_quantize_halfway_and_rounding_cases(orc):
     assert orc.quantize(np.float32(-3e9), r) == 2**31 - 1   # INT_MIN - 1 wraps (sub.s32)
     assert orc.quantize(np.float32("nan"), r) == -1
     assert orc.quantize(np.float32("inf"), r) == 2**31 - 1
+    # the edges of the saturating conversion (PTX cvt.rzi.s32.f32): 2^31 itself is already out of
+    # range and saturates, the largest float below it converts as it is; -2^31 is in range
+    assert orc.quantize(np.float32(2147483648.0), r) == 2**31 - 1
+    assert orc.quantize(np.float32(2147483520.0), r) == 2147483520
+    assert orc.quantize(np.float32(-2147483648.0), r) == 2**31 - 1   # INT_MIN, minus the s = 1 of a negative d, wraps
 
 
 def test_quantize_matches_float32_model_and_bound(orc):
@@ -255,6 +260,50 @@ def test_out_of_bound_rule(orc, gen):
     assert not d[501:].any()
     out = orc.decompress(s, n, eb, cmp_size=cut)
     assert not out[501 * 32:].any()
+
+
+def test_out_of_bound_rule_at_the_boundary(orc, gen):
+    """GSZ.cu:908 compares with >=: a block whose payload starts exactly at the stated size is
+    skipped, one that starts a byte below it is read in full -- in the decoder and in the sums'
+    decoding of their incoming stream (HomComp/src/homcomp.cu:3081-3084)."""
+    n = 32768
+    x = gen.uniform_np(n, 5)
+    eb = np.float32(1e-3)
+    s, ofs = orc.compress(x, eb, want_offsets=True)
+    full = orc.decode_deltas(s, n).reshape(-1, 32)
+    for b in (1, 2, 700, 1023):
+        at = int(ofs[b])
+        assert int(ofs[b + 1]) > at, "a block with payload"
+        d = orc.decode_deltas(s, n, cmp_size=at).reshape(-1, 32)          # block b starts at the stated size
+        assert np.array_equal(d[:b], full[:b]) and not d[b:].any(), b
+        d = orc.decode_deltas(s, n, cmp_size=at + 1).reshape(-1, 32)      # ... a byte below it
+        assert np.array_equal(d[:b + 1], full[:b + 1]) and not d[b + 1:].any(), b
+        # the same through a sum with an all-zero local operand: what was decoded is re-encoded
+        zeros = np.zeros(n, np.int32)
+        for cut, upto in ((at, b), (at + 1, b + 1)):
+            want = full.copy()
+            want[upto:] = 0
+            assert np.array_equal(orc.hom_sum_i32(s, zeros, cmp_in_size=cut), orc.encode_deltas(want.reshape(-1))), (b, cut)
+
+
+def test_plane_count_is_capped_at_31(orc):
+    """A magnitude of 2^31 (only a saturated quantisation produces it) has 32 bits, which the
+    five-bit field of the header byte cannot hold: this implementation, like its oracle, caps the
+    plane count at 31 and stays self-consistent (a deviation by choice: the reference writes 32
+    into the byte, i.e. zero planes and a bit of the outlier-width field, which its own decoder
+    then misreads)."""
+    d = np.zeros(32, np.int32)
+    d[3] = -2**31
+    hdr, payload = orc.block_encode(d)
+    assert hdr & 0x1f == 31 and len(payload) == orc.block_size_from_header(hdr)
+    back = orc.block_decode(hdr, payload)
+    assert back[3] == 0 and not back.any()          # bit 31 of the magnitude is not stored: the value decodes to -0 = 0
+    d[0] = -2**31                                   # as the block's first element: four outlier bytes hold all 32 bits
+    d[3] = 5
+    hdr, payload = orc.block_encode(d)
+    assert hdr >> 7 == 1 and (hdr >> 5) & 3 == 3 and hdr & 0x1f == 3
+    back = orc.block_decode(hdr, payload)
+    assert back[0] == -2**31 and back[3] == 5
 
 
 # ------------------------------------------------------------------ homomorphic sums
