@@ -134,8 +134,9 @@ __device__ __forceinline__ uint32_t planes_of(uint32_t m)
     return b > 31u ? 31u : b;
 }
 
-// HomComp/src/GSZ.cu:795-802: payload bytes implied by a header byte.
-__device__ __forceinline__ uint32_t size_from_header(uint32_t h)
+// HomComp/src/GSZ.cu:795-802: payload bytes implied by a header byte.  (The kernels use the
+// byte-parallel forms below; this one is what they are checked against, at compile time.)
+__device__ __forceinline__ constexpr uint32_t size_from_header(uint32_t h)
 {
     uint32_t F = h & 0x1fu;
     uint32_t ob = ((h >> 5) & 3u) + 1u;
@@ -340,7 +341,7 @@ __device__ __forceinline__ void unpack_low4(const uint8_t *stage, uint32_t base,
 
 // Sizes (size_from_header) and digests (header_digest, below) of two header bytes at once, a
 // byte each in the results: the same byte-parallel arithmetic as add_sizes_from_4_headers.
-__device__ __forceinline__ void sizes_and_digests_of_2_headers(uint32_t w, uint32_t &sizes, uint32_t &digests)
+__device__ __forceinline__ constexpr void sizes_and_digests_of_2_headers(uint32_t w, uint32_t &sizes, uint32_t &digests)
 {
     const uint32_t F = w & 0x1f1fu;
     const uint32_t sel = (w >> 7) & 0x0101u;
@@ -352,12 +353,26 @@ __device__ __forceinline__ void sizes_and_digests_of_2_headers(uint32_t w, uint3
 
 // What the decoder needs of a header byte, in one byte: bits 0-4 the plane count F, bits 5-7 the
 // number of outlier bytes (0 in plain mode, 1-4 in outlier mode).  0 for a block without payload.
-__device__ __forceinline__ uint32_t header_digest(uint32_t h)
+__device__ __forceinline__ constexpr uint32_t header_digest(uint32_t h)
 {
     const uint32_t F = h & 0x1fu;
     const uint32_t ob = (h & 0x80u) ? ((h >> 5) & 3u) + 1u : 0u;
     return F | (ob << 5);
 }
+
+// every header byte, in either place of a pair, against the two definitions a byte at a time
+__device__ __forceinline__ constexpr bool pairs_of_headers_agree_with_single_ones()
+{
+    for (uint32_t h = 0; h < 256u; ++h) {
+        const uint32_t other = (h * 167u + 13u) & 0xffu;
+        uint32_t sizes = 0, digests = 0;
+        sizes_and_digests_of_2_headers(h | (other << 8), sizes, digests);
+        if ((sizes & 0xffu) != size_from_header(h) || (sizes >> 8) != size_from_header(other)) return false;
+        if ((digests & 0xffu) != header_digest(h) || (digests >> 8) != header_digest(other)) return false;
+    }
+    return true;
+}
+static_assert(pairs_of_headers_agree_with_single_ones(), "sizes_and_digests_of_2_headers");
 
 // (a ^ b) + c in one instruction
 __device__ __forceinline__ uint32_t xor_add(uint32_t a, uint32_t b, uint32_t c)
