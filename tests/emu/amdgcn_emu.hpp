@@ -80,6 +80,10 @@ struct emu_wave {
     uint64_t slot[2][64];
     std::vector<emu_store> log;
     void *main_sp;             // the wave thread's own stack pointer while its lanes run
+    const uint8_t *stacks;     // the lanes' stacks, one after the other, stack_bytes each
+    size_t stack_bytes;
+    const void *main_stack;    // the wave thread's own stack (known to a sanitizer build only)
+    size_t main_stack_bytes;
     const void *kernel;        // std::function<void()> of the launch
 };
 extern thread_local emu_wave *emu_wave_of_thread;
@@ -131,6 +135,27 @@ inline void emu_ordered_store32(void *addr, uint32_t value, uint32_t index) { em
 
 // saves the callee-saved registers and the stack pointer of the running lane, takes up another's
 extern "C" void emu_switch(void **save_sp, void *load_sp);
+// The same with the notices an AddressSanitizer build of the model needs about stacks that change
+// under it (`bottom`, `bytes`: the stack that is switched to; `leaving`: the running lane never comes back).
+#if defined(__has_feature)
+#if __has_feature(address_sanitizer)
+#define EMU_ASAN 1
+extern "C" void __sanitizer_start_switch_fiber(void **fake_stack_save, const void *bottom, size_t size);
+extern "C" void __sanitizer_finish_switch_fiber(void *fake_stack_save, const void **bottom_old, size_t *size_old);
+#endif
+#endif
+inline void emu_switch_stacks(void **save_sp, void *load_sp, const void *bottom, size_t bytes, bool leaving = false)
+{
+#ifdef EMU_ASAN
+    void *fake = nullptr;
+    __sanitizer_start_switch_fiber(leaving ? nullptr : &fake, bottom, bytes);
+    emu_switch(save_sp, load_sp);
+    __sanitizer_finish_switch_fiber(fake, nullptr, nullptr);
+#else
+    (void)bottom, (void)bytes, (void)leaving;
+    emu_switch(save_sp, load_sp);
+#endif
+}
 // gives way to the next lane of the wave that has not left the kernel
 inline void emu_next_lane(emu_wave *w)
 {
@@ -146,7 +171,7 @@ inline void emu_next_lane(emu_wave *w)
         abort();
     }
     emu_cur = next;
-    emu_switch(&me->sp, next->sp);
+    emu_switch_stacks(&me->sp, next->sp, w->stacks + (size_t)next->lane * w->stack_bytes, w->stack_bytes, me->done);
 }
 // the last lane to arrive lets the meeting go: the logged stores are carried out in program order first
 inline void emu_release(emu_wave *w)

@@ -81,12 +81,23 @@ const size_t emu_lane_stack = 1 << 20;   // per lane; only the pages a lane touc
 extern "C" inline void emu_lane_entry()
 {
     emu_wave *w = emu_wave_of_thread;
+#ifdef EMU_ASAN
+    {   // first time on this stack; the wave's first lane learns the thread's own stack from it
+        const void *from = nullptr;
+        size_t from_bytes = 0;
+        __sanitizer_finish_switch_fiber(nullptr, &from, &from_bytes);
+        if (!w->main_stack) {
+            w->main_stack = from;
+            w->main_stack_bytes = from_bytes;
+        }
+    }
+#endif
     (*(const std::function<void()> *)w->kernel)();
     emu_lane_ctx *me = emu_cur;
     me->done = true;
     w->live--;
     if (w->live == 0) {
-        emu_switch(&me->sp, w->main_sp);   // the wave is through; does not come back
+        emu_switch_stacks(&me->sp, w->main_sp, w->main_stack, w->main_stack_bytes, true);   // the wave is through; does not come back
     }
     if (w->arrived == w->live) emu_release(w);   // the others were waiting for this lane only
     emu_next_lane(w);                             // does not come back either
@@ -100,6 +111,7 @@ inline void *emu_wave_main(void *arg)
     emu_wave *w = new emu_wave;
     emu_wave_of_thread = w;
     w->kernel = k->kernel;
+    w->stack_bytes = emu_lane_stack;
     w->count = k->threads - 64 * s->index < 64 ? k->threads - 64 * s->index : 64;
     uint8_t *stacks = (uint8_t *)mmap(nullptr, 64 * emu_lane_stack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
     if (stacks == MAP_FAILED) {
@@ -107,6 +119,7 @@ inline void *emu_wave_main(void *arg)
         _exit(3);
     }
     for (unsigned l = 0; l < 64; ++l) mprotect(stacks + l * emu_lane_stack, emu_page, PROT_NONE);   // a lane that outgrows its stack faults
+    w->stacks = stacks;
     for (unsigned i = k->first; i < k->blocks; i += k->step) {
         if (s->index == 0) {
             blockIdx.x = i % k->grid_x;
@@ -134,7 +147,8 @@ inline void *emu_wave_main(void *arg)
         w->log.clear();
         pthread_barrier_wait(&emu_block_barrier);
         emu_cur = &w->lanes[0];
-        emu_switch(&w->main_sp, w->lanes[0].sp);   // back here when the wave's last lane has left the kernel
+        w->main_stack = nullptr;
+        emu_switch_stacks(&w->main_sp, w->lanes[0].sp, stacks, emu_lane_stack);   // back here when the wave's last lane has left the kernel
         pthread_barrier_wait(&emu_block_barrier);
     }
     munmap(stacks, 64 * emu_lane_stack);
