@@ -91,6 +91,16 @@ extern thread_local emu_lane_ctx *emu_cur;   // the lane that is running on this
 #define threadIdx (emu_cur->tid)
 #define emu_lane (emu_cur->lane)
 extern pthread_barrier_t emu_block_barrier;   // of the workgroup's wave threads
+// Dynamic LDS: the array that stands for it has the size of the largest launch; what lies beyond
+// the size of the launch under way holds a pattern that must still be there when a workgroup ends.
+extern uint8_t *emu_dynamic_lds;          // where the running kernel's array is (a kernel with one says so)
+extern size_t emu_dynamic_lds_bytes;      // of the launch under way
+inline void emu_note_dynamic_lds(uint8_t *array)
+{
+    // the first lane of the workgroup to come by lays the pattern (nothing has used the array yet)
+    if (__sync_bool_compare_and_swap(&emu_dynamic_lds, (uint8_t *)nullptr, array))
+        memset(array + emu_dynamic_lds_bytes, 0xD5, EMU_DYN_LDS - emu_dynamic_lds_bytes);
+}
 
 // Every access a kernel makes to "device memory" must fall into a registered allocation; the
 // first one that does not is reported with its address and aborts the run.

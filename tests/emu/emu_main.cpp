@@ -77,10 +77,10 @@ struct Launch {
     const void *args;
 };
 
-void run_grid(const Launch &l, unsigned gx, unsigned gy, unsigned threads)
+void run_grid(const Launch &l, unsigned gx, unsigned gy, unsigned threads, size_t dyn_lds = 0)
 {
     const std::function<void()> body = [=]() { l.kernel(l.args); };
-    if (!emu_run_grid(body, emu_dim3(gx, gy), emu_dim3(threads))) exit(4);
+    if (!emu_run_grid(body, emu_dim3(gx, gy), emu_dim3(threads), dyn_lds)) exit(4);
 }
 
 template <int NIN, int LOCAL, int OUT, int BITPLANE>
@@ -284,7 +284,7 @@ int main(int argc, char **argv)
         l.kernel = kind == 2 ? wave_kernel<2, hc::kLocalNone, hc::kOutStream, hc::kPlanesWide> : wave_kernel<2, hc::kLocalNone, hc::kOutStream, hc::kPlanesFew>;
     else
         return 1;
-    run_grid(l, groups + (enc ? 1u : 0u), 1, 256);
+    run_grid(l, groups + (enc ? 1u : 0u), 1, 256, enc ? 4u * (size_t)budget : 0u);   // as launch_wave asks for it
     if (*p.error) {
         fprintf(stderr, "EMU: the kernels raised the error word (0x%x)\n", *p.error);
         return 5;

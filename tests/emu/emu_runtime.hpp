@@ -14,7 +14,9 @@
 // One translation unit of a program defines EMU_DEFINE_GLOBALS before including this.
 #pragma once
 
+#include <signal.h>
 #include <sys/mman.h>
+#include <sys/prctl.h>
 #include <sys/wait.h>
 #include <unistd.h>
 
@@ -145,11 +147,21 @@ inline void *emu_wave_main(void *arg)
         w->arrived = 0;
         w->gen = 0;
         w->log.clear();
+        if (s->index == 0) emu_dynamic_lds = nullptr;
         pthread_barrier_wait(&emu_block_barrier);
         emu_cur = &w->lanes[0];
         w->main_stack = nullptr;
         emu_switch_stacks(&w->main_sp, w->lanes[0].sp, stacks, emu_lane_stack);   // back here when the wave's last lane has left the kernel
         pthread_barrier_wait(&emu_block_barrier);
+        if (s->index == 0 && emu_dynamic_lds) {
+            // nothing was written beyond the dynamic LDS the launch asked for (the pattern emu_note_dynamic_lds laid)
+            for (uint8_t *b = emu_dynamic_lds + emu_dynamic_lds_bytes; b != emu_dynamic_lds + EMU_DYN_LDS; ++b)
+                if (*b != 0xD5u) {
+                    fprintf(stderr, "EMU: block %u wrote %zu bytes beyond its %zu bytes of dynamic LDS\n", i,
+                            (size_t)(b - emu_dynamic_lds) - emu_dynamic_lds_bytes + 1, emu_dynamic_lds_bytes);
+                    _exit(5);
+                }
+        }
     }
     munmap(stacks, 64 * emu_lane_stack);
     delete w;
@@ -188,13 +200,15 @@ inline unsigned emu_resident_limit()
     const int v = e ? atoi(e) : 48;
     return v < 1 ? 1u : (unsigned)v;
 }
-inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu_dim3 block)
+inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu_dim3 block, size_t dyn_lds = EMU_DYN_LDS)
 {
     const emu_locked lock(&emu_launch_lock);   // one launch at a time, whichever host thread makes it
+    emu_dynamic_lds_bytes = dyn_lds;
     gridDim = grid;
     blockDim = block;
     const unsigned n = grid.x * grid.y * grid.z, limit = emu_resident_limit(), workers = n < limit ? n : limit;
     pid_t *kids = new pid_t[workers];
+    const pid_t parent = getpid();
     unsigned started = 0;
     bool ok = true;
     fflush(nullptr);
@@ -206,6 +220,9 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
             break;
         }
         if (k == 0) {
+            // a worker does not outlive the program that launched it (one that was killed at a time limit, say)
+            prctl(PR_SET_PDEATHSIG, SIGKILL);
+            if (getppid() != parent) _exit(6);
             emu_worker w{&kernel, block.x, i, workers, n, grid.x};
             emu_run_worker(w);
             fflush(nullptr);
@@ -249,7 +266,7 @@ inline void emu_launch(K kernel, emu_dim3 grid, emu_dim3 block, size_t dyn_lds, 
         return;
     }
     const std::function<void()> body = [=]() { kernel(args...); };
-    if (!emu_run_grid(body, grid, block)) emu_last_error = hipErrorLaunchFailure;
+    if (!emu_run_grid(body, grid, block, dyn_lds)) emu_last_error = hipErrorLaunchFailure;
 }
 #define hipLaunchKernelGGL(kernel, grid, block, dyn, stream, ...) emu_launch(kernel, grid, block, dyn, stream, __VA_ARGS__)
 
@@ -381,6 +398,8 @@ emu_dim3 blockIdx, gridDim, blockDim;
 thread_local emu_wave *emu_wave_of_thread = nullptr;
 thread_local emu_lane_ctx *emu_cur = nullptr;
 pthread_barrier_t emu_block_barrier;
+uint8_t *emu_dynamic_lds = nullptr;
+size_t emu_dynamic_lds_bytes = 0;
 emu_alloc emu_allocs[8192];
 int emu_n_allocs = 0;
 thread_local hipError_t emu_last_error = hipSuccess;

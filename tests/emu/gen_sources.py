@@ -37,7 +37,7 @@ DEVICE_EDITS = [
     ("        if (w <= o.F) store_u32_any(at + 4u * w, o.w[w]);", "        if (w <= o.F) emu_ordered_store32(at + 4u * w, o.w[w], kWideChunks + 1 + w);"),
 ]
 KERNEL_EDITS = [
-    ("    extern __shared__ __align__(16) uint8_t s_dyn[];", "    static __attribute__((aligned(16), section(\"emu_lds\"))) uint8_t s_dyn[EMU_DYN_LDS];"),
+    ("    extern __shared__ __align__(16) uint8_t s_dyn[];", "    static __attribute__((aligned(16), section(\"emu_lds\"))) uint8_t s_dyn[EMU_DYN_LDS];\n    emu_note_dynamic_lds(s_dyn);"),
     ('            if constexpr (kSlicedLocal) asm volatile("" : "+v"(fresh_lane));', ""),
     # A wave's LDS instructions take effect in the order of the program, for all its lanes: what the lanes packed is
     # in the stage when the instructions that move it elsewhere read it.  Lanes that are threads have to meet for that.
