@@ -41,6 +41,32 @@ def gen():
     return OnTheModel()
 
 
+def _load_file(name, path):
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(name, path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.fixture(scope="session")
+def emu_sources():
+    """tests/emu/gen_sources.py: builds the CPU execution model's programs and library from the
+    product's source; the tests that need it are skipped where the ROCm clang++ is missing."""
+    mod = _load_file("emu_gen_sources", os.path.join(ROOT, "tests", "emu", "gen_sources.py"))
+    if not os.path.exists(mod.CLANG):
+        pytest.skip("the ROCm clang++ that the host build of the device code needs is not installed")
+    os.environ.setdefault("EMU_CUS", "3")
+    return mod
+
+
+@pytest.fixture(scope="session")
+def emulated(emu_sources):
+    """(the product's binding bound to libhomcomp_emu.so, tests/emu/harness.py)"""
+    harness = _load_file("emu_harness", os.path.join(ROOT, "tests", "emu", "harness.py"))
+    return harness.load_binding(emu_sources.build_library()), harness
+
+
 def _cpu_model():
     """HOMCOMP_CPU_MODEL=1 points the gpu-marked tests at the library built for the host against
     the CPU execution model (tests/emu) instead of the GPU: the same binding bound to
@@ -50,17 +76,10 @@ def _cpu_model():
     if os.environ.get("HOMCOMP_CPU_MODEL", "0") in ("", "0"):
         return None
     if "binding" not in _model:
-        import importlib.util
-
-        def load(name, path):
-            spec = importlib.util.spec_from_file_location(name, path)
-            mod = importlib.util.module_from_spec(spec)
-            spec.loader.exec_module(mod)
-            return mod
         here = os.path.join(ROOT, "tests", "emu")
-        harness = load("emu_harness", os.path.join(here, "harness.py"))
+        harness = _load_file("emu_harness", os.path.join(here, "harness.py"))
         os.environ.setdefault("EMU_CUS", "5")
-        _model["binding"] = harness.load_binding(load("emu_gen_sources", os.path.join(here, "gen_sources.py")).build_library())
+        _model["binding"] = harness.load_binding(_load_file("emu_gen_sources", os.path.join(here, "gen_sources.py")).build_library())
         _model["torch"] = harness.EmuTorch(_model["binding"].lib())
     return _model
 

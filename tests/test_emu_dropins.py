@@ -3,7 +3,6 @@ GSZ_entry with the plain and host-pointer entries, the ring all-reduce with its 
 threads, the evaluator) built for the host against the execution model of tests/emu and linked
 with libhomcomp_emu.so, checked by the very functions the gpu-marked tests use, at sizes the
 model finishes in seconds."""
-import importlib.util
 import os
 import sys
 
@@ -17,14 +16,8 @@ import test_gpu_shim  # noqa: E402
 
 
 @pytest.fixture(scope="module")
-def programs():
-    spec = importlib.util.spec_from_file_location("emu_gen_sources", os.path.join(HERE, "emu", "gen_sources.py"))
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
-    if not os.path.exists(mod.CLANG):
-        pytest.skip("the ROCm clang++ that the host build needs is not installed")
-    os.environ.setdefault("EMU_CUS", "3")
-    return mod.build_programs()
+def programs(emu_sources):
+    return emu_sources.build_programs()
 
 
 @pytest.mark.parametrize("n", [32768 * 2 + 100, 4096])

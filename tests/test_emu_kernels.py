@@ -7,24 +7,17 @@ short; and, through the guard pages and the checked buffer descriptors, that no 
 its buffer.  It does not cover the compiler, timing or the memory model of the hardware: parity
 on the GPU stays with the gpu-marked tests.
 """
-import importlib.util
 import os
 import subprocess
 
 import numpy as np
 import pytest
 
-HERE = os.path.dirname(os.path.abspath(__file__))
 
 
 @pytest.fixture(scope="module")
-def emu(tmp_path_factory):
-    spec = importlib.util.spec_from_file_location("emu_gen_sources", os.path.join(HERE, "emu", "gen_sources.py"))
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
-    if not os.path.exists(mod.CLANG):
-        pytest.skip("the ROCm clang++ that the host build of the device code needs is not installed")
-    return Emu(mod.build(), str(tmp_path_factory.mktemp("emu")))
+def emu(emu_sources, tmp_path_factory):
+    return Emu(emu_sources.build(), str(tmp_path_factory.mktemp("emu")))
 
 
 class Emu:

@@ -8,7 +8,6 @@ tile offsets, the allocation-free entry, the bounded waits and their recovery.  
 streams that run side by side and the hardware itself stay with the gpu-marked tests.
 """
 import ctypes as C
-import importlib.util
 import os
 import sys
 
@@ -18,24 +17,6 @@ import pytest
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
 from gpu_util import Gpu, first_diff  # noqa: E402
-
-
-def _load(name, path):
-    spec = importlib.util.spec_from_file_location(name, path)
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
-    return mod
-
-
-@pytest.fixture(scope="module")
-def emulated():
-    gen_sources = _load("emu_gen_sources", os.path.join(HERE, "emu", "gen_sources.py"))
-    if not os.path.exists(gen_sources.CLANG):
-        pytest.skip("the ROCm clang++ that the host build of the library needs is not installed")
-    harness = _load("emu_harness", os.path.join(HERE, "emu", "harness.py"))
-    os.environ.setdefault("EMU_CUS", "3")
-    binding = harness.load_binding(gen_sources.build_library())
-    return binding, harness
 
 
 @pytest.fixture()

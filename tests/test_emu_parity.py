@@ -6,7 +6,6 @@ zero blocks, special values, empty input, truncated sizes, unaligned stream poin
 lengths, random mixtures; the plain codec's tests, the tile offsets' and the allocation-free
 entry's argument checks likewise (tests/test_gpu_plain.py, test_gpu_tile_offsets.py,
 test_zz_no_alloc.py)."""
-import importlib.util
 import os
 import sys
 
@@ -19,23 +18,6 @@ import test_gpu_plain as plain  # noqa: E402
 import test_gpu_tile_offsets as tile_offsets  # noqa: E402
 import test_zz_no_alloc as no_alloc  # noqa: E402
 from gpu_util import Gpu  # noqa: E402
-
-
-def _load(name, path):
-    spec = importlib.util.spec_from_file_location(name, path)
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
-    return mod
-
-
-@pytest.fixture(scope="module")
-def emulated():
-    gen_sources = _load("emu_gen_sources", os.path.join(HERE, "emu", "gen_sources.py"))
-    if not os.path.exists(gen_sources.CLANG):
-        pytest.skip("the ROCm clang++ that the host build of the library needs is not installed")
-    harness = _load("emu_harness", os.path.join(HERE, "emu", "harness.py"))
-    os.environ.setdefault("EMU_CUS", "3")
-    return harness.load_binding(gen_sources.build_library()), harness
 
 
 @pytest.fixture()
