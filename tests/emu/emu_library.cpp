@@ -21,4 +21,22 @@ int emu_free_buffer(void *p) { return emu_device_free(p) ? 0 : 1; }
 
 int emu_live_allocations(void) { return emu_n_allocs; }
 
+// bytes of "device memory" in use (what a free-memory query would be taken from)
+size_t emu_live_bytes(void)
+{
+    const emu_locked lock(&emu_alloc_lock);
+    size_t total = 0;
+    for (int i = 0; i < emu_n_allocs; ++i) total += emu_allocs[i].hi - emu_allocs[i].lo;
+    return total;
+}
+
+// Graph capture for the harness: between begin and end every launch the library makes is recorded
+// instead of run; a replay runs the recorded launches in order, with their recorded arguments,
+// on whatever the buffers hold then.
+void *emu_graph_begin_capture(void) { return emu_capture_begin(); }
+void *emu_graph_end_capture(void) { return emu_capture_end(); }
+int emu_graph_launch(void *graph) { return emu_graph_replay((emu_graph *)graph) ? 0 : 1; }
+int emu_graph_launches(void *graph) { return (int)((emu_graph *)graph)->launches.size(); }
+void emu_graph_destroy(void *graph) { delete (emu_graph *)graph; }
+
 }  // extern "C"

@@ -9,7 +9,10 @@
 //                   forked process per workgroup, all alive together, 64 threads per wave
 //   the device      EMU_CUS compute units (environment, default 3) with 160 KB of LDS each; the
 //                   occupancy query divides that by a kernel's LDS and caps the result at 4
-//   graph capture   does not exist here: no stream is ever capturing
+//   graph capture   one capture at a time, of every stream at once (emu_capture_begin / _end, for
+//                   the test harness): launches are recorded with their arguments instead of run,
+//                   and run in order at every replay; an allocation, a copy or a memset while a
+//                   capture is under way ends the run with a report (the library must not make one)
 //
 // One translation unit of a program defines EMU_DEFINE_GLOBALS before including this.
 #pragma once
@@ -21,6 +24,7 @@
 #include <unistd.h>
 
 #include <functional>
+#include <vector>
 
 #include "amdgcn_emu.hpp"
 
@@ -257,6 +261,38 @@ inline hipError_t hipGetLastError()
     return e;
 }
 
+// ---- graph capture
+struct emu_graph {
+    std::vector<std::function<bool()>> launches;
+};
+extern emu_graph *emu_capturing;            // the graph under construction, if any
+extern unsigned long long emu_capture_id;   // of that capture (unique per capture)
+inline void emu_not_while_capturing(const char *what)
+{
+    if (emu_capturing) {
+        fprintf(stderr, "EMU: %s while a graph is being captured\n", what);
+        abort();
+    }
+}
+inline emu_graph *emu_capture_begin()
+{
+    emu_not_while_capturing("a second capture");
+    ++emu_capture_id;
+    return emu_capturing = new emu_graph;
+}
+inline emu_graph *emu_capture_end()
+{
+    emu_graph *g = emu_capturing;
+    emu_capturing = nullptr;
+    return g;
+}
+inline bool emu_graph_replay(emu_graph *g)
+{
+    for (const std::function<bool()> &launch : g->launches)
+        if (!launch()) return false;
+    return true;
+}
+
 // hipLaunchKernelGGL(kernel, grid, block, dynamic LDS, stream, arguments...)
 template <typename K, typename... A>
 inline void emu_launch(K kernel, emu_dim3 grid, emu_dim3 block, size_t dyn_lds, hipStream_t, A... args)
@@ -266,12 +302,17 @@ inline void emu_launch(K kernel, emu_dim3 grid, emu_dim3 block, size_t dyn_lds, 
         return;
     }
     const std::function<void()> body = [=]() { kernel(args...); };
+    if (emu_capturing) {
+        emu_capturing->launches.push_back([=]() { return emu_run_grid(body, grid, block, dyn_lds); });
+        return;
+    }
     if (!emu_run_grid(body, grid, block, dyn_lds)) emu_last_error = hipErrorLaunchFailure;
 }
 #define hipLaunchKernelGGL(kernel, grid, block, dyn, stream, ...) emu_launch(kernel, grid, block, dyn, stream, __VA_ARGS__)
 
 inline hipError_t hipMalloc(void **p, size_t bytes)
 {
+    emu_not_while_capturing("hipMalloc");
     *p = emu_device_alloc_named(bytes, "hipMalloc");
     if (*p) memset(*p, 0xB6, bytes);   // fresh device memory is not zero
     return *p ? hipSuccess : hipErrorOutOfMemory;
@@ -291,6 +332,7 @@ inline hipError_t hipHostMalloc(void **p, size_t bytes, unsigned)
 inline hipError_t hipHostFree(void *p) { return hipFree(p); }
 inline hipError_t hipMemset(void *p, int v, size_t bytes)
 {
+    emu_not_while_capturing("a memset (a memset node in a graph has given wrong results on replays; the library fills with a kernel)");
     emu_check(p, bytes, "hipMemset");
     memset(p, v, bytes);
     return hipSuccess;
@@ -298,6 +340,7 @@ inline hipError_t hipMemset(void *p, int v, size_t bytes)
 enum hipMemcpyKind { hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
 inline hipError_t hipMemcpy(void *dst, const void *src, size_t bytes, hipMemcpyKind kind)
 {
+    emu_not_while_capturing("a copy");
     // the side that is device memory must lie inside an allocation
     if (kind == hipMemcpyHostToDevice || kind == hipMemcpyDeviceToDevice) emu_check(dst, bytes, "hipMemcpy (destination)");
     if (kind == hipMemcpyDeviceToHost || kind == hipMemcpyDeviceToDevice) emu_check(src, bytes, "hipMemcpy (source)");
@@ -344,8 +387,8 @@ inline hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) { return
 enum hipStreamCaptureStatus { hipStreamCaptureStatusNone, hipStreamCaptureStatusActive, hipStreamCaptureStatusInvalidated };
 inline hipError_t hipStreamGetCaptureInfo(hipStream_t, hipStreamCaptureStatus *status, unsigned long long *id)
 {
-    *status = hipStreamCaptureStatusNone;
-    if (id) *id = 0;
+    *status = emu_capturing ? hipStreamCaptureStatusActive : hipStreamCaptureStatusNone;
+    if (id) *id = emu_capturing ? emu_capture_id : 0;
     return hipSuccess;
 }
 // A kernel's LDS is not known to this model: every kernel is taken to have the static LDS of the
@@ -400,6 +443,8 @@ thread_local emu_lane_ctx *emu_cur = nullptr;
 pthread_barrier_t emu_block_barrier;
 uint8_t *emu_dynamic_lds = nullptr;
 size_t emu_dynamic_lds_bytes = 0;
+emu_graph *emu_capturing = nullptr;
+unsigned long long emu_capture_id = 0;
 emu_alloc emu_allocs[8192];
 int emu_n_allocs = 0;
 thread_local hipError_t emu_last_error = hipSuccess;

@@ -34,16 +34,104 @@ def load_binding(library_path: str):
     return mod
 
 
-class _Host:
-    """What torch.from_numpy returns, as far as the helpers go: something with .cuda()."""
-
-    def __init__(self, dev, array):
-        self._dev, self._array = dev, np.ascontiguousarray(array)
+class _Host(torch.Tensor):
+    """What torch.from_numpy returns here: a CPU tensor over the array whose .cuda() copies it into
+    the model's device memory."""
 
     def cuda(self):
-        t = self._dev.empty(self._array.shape, dtype=torch.from_numpy(self._array).dtype)
-        t.copy_(torch.from_numpy(self._array))
+        plain = self.as_subclass(torch.Tensor)
+        t = self._emu_device.empty(tuple(plain.shape), dtype=plain.dtype)
+        t.copy_(plain)
         return t
+
+
+class _Stream:
+    """Every stream is the one synchronous stream of the model."""
+    cuda_stream = 0
+
+    def wait_stream(self, other):
+        pass
+
+    def synchronize(self):
+        pass
+
+
+class _Graph:
+    def __init__(self, library):
+        self._lib, self._h = library, None
+
+    def replay(self):
+        assert self._h, "a graph that was never captured"
+        assert self._lib.emu_graph_launch(self._h) == 0, "a launch of the graph failed"
+
+    def __del__(self):
+        if self._h:
+            self._lib.emu_graph_destroy(self._h)
+
+
+class _Capture:
+    def __init__(self, library, graph):
+        self._lib, self._graph = library, graph
+
+    def __enter__(self):
+        self._lib.emu_graph_begin_capture()
+        return self
+
+    def __exit__(self, *exc):
+        self._graph._h = self._lib.emu_graph_end_capture()
+        return False
+
+
+class _Nothing:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+class _Cuda:
+    """torch.cuda, as far as the tests use it: streams (all the one synchronous stream), graphs
+    (the model's record-and-replay of launches), the free-memory query (from the model's list of
+    allocations)."""
+    TOTAL = 288 << 30
+
+    def __init__(self, library):
+        self._lib = library
+        for name in ("emu_graph_begin_capture", "emu_graph_end_capture"):
+            getattr(library, name).restype = C.c_void_p
+        library.emu_graph_launch.argtypes = [C.c_void_p]
+        library.emu_graph_destroy.argtypes = [C.c_void_p]
+        library.emu_live_bytes.restype = C.c_size_t
+
+    def synchronize(self):
+        pass
+
+    def empty_cache(self):
+        pass
+
+    def Stream(self):
+        return _Stream()
+
+    def current_stream(self):
+        return _Stream()
+
+    def stream(self, s):
+        return _Nothing()
+
+    def CUDAGraph(self):
+        return _Graph(self._lib)
+
+    def graph(self, graph, stream=None):
+        return _Capture(self._lib, graph)
+
+    def mem_get_info(self):
+        return self.TOTAL - int(self._lib.emu_live_bytes()), self.TOTAL
+
+    def memory_reserved(self):
+        return int(self._lib.emu_live_bytes())
+
+    memory_allocated = memory_reserved
 
 
 class EmuTorch:
@@ -52,15 +140,13 @@ class EmuTorch:
     uint8, int32, int64, float32 = torch.uint8, torch.int32, torch.int64, torch.float32
     equal = staticmethod(torch.equal)
 
-    class cuda:
-        synchronize = staticmethod(lambda: None)
-
     def __init__(self, library):
         self._lib = library
         self._lib.emu_alloc_buffer.restype = C.c_void_p
         self._lib.emu_alloc_buffer.argtypes = [C.c_size_t, C.c_size_t]
         self._lib.emu_free_buffer.argtypes = [C.c_void_p]
         self._live = []
+        self.cuda = _Cuda(library)
 
     def empty(self, shape, dtype=torch.float32, device="cuda"):
         assert device == "cuda"
@@ -87,7 +173,9 @@ class EmuTorch:
         return t
 
     def from_numpy(self, array):
-        return _Host(self, array)
+        host = torch.from_numpy(np.ascontiguousarray(array)).as_subclass(_Host)
+        host._emu_device = self
+        return host
 
     def release(self):
         """Frees every buffer handed out (tensors over them must not be touched afterwards)."""

@@ -1,11 +1,12 @@
-"""The gpu-marked parity tests, all but the three that need graphs or streams side by side, run as
-they are (tests/test_gpu_parity.py, the same functions) with the library built for the host
+"""The gpu-marked parity tests, all but the two that need streams or host threads side by side, run
+as they are (tests/test_gpu_parity.py, the same functions) with the library built for the host
 (libhomcomp_emu.so, tests/emu) behind the same binding and helper: crafted streams of every plane
 count, mode and outlier width, the bit-plane paths, payloads of random bytes under valid headers,
 zero blocks, special values, empty input, truncated sizes, unaligned stream pointers, ragged
-lengths, random mixtures; the plain codec's tests, the tile offsets' and the allocation-free
-entry's argument checks likewise (tests/test_gpu_plain.py, test_gpu_tile_offsets.py,
-test_zz_no_alloc.py)."""
+lengths, random mixtures, a graph replayed with eager calls between the replays; the plain
+codec's tests, the tile offsets' (a recorded chain of ring steps among them) and the
+allocation-free entry's (arguments, nothing allocated, recorded into a graph) likewise
+(tests/test_gpu_plain.py, test_gpu_tile_offsets.py, test_zz_no_alloc.py)."""
 import os
 import sys
 
@@ -153,3 +154,21 @@ def test_offsets_written_and_taken(world, orc, gen, kind, n, rel):
 # ---- tests/test_zz_no_alloc.py
 def test_static_entry_limits_and_arguments(world):
     no_alloc.test_static_entry_limits_and_arguments(world[1], world[2])
+
+
+# ---- graphs: the model records the launches a capture makes and runs them again at every replay; an
+#      allocation, a copy or a memset while a capture is under way would end the run with a report
+def test_graph_replay(world, orc, gen):
+    parity.test_graph_replay(world[1], world[2], orc, gen)
+
+
+def test_ring_steps_recorded_with_offsets(world, orc, gen):
+    tile_offsets.test_ring_steps_recorded_with_offsets(world[1], world[2], orc, gen)
+
+
+def test_static_entry_in_a_graph(world, orc, gen):
+    no_alloc.test_static_entry_in_a_graph(world[1], world[2], orc, gen)
+
+
+def test_static_entry_allocates_nothing(world, orc, gen):
+    no_alloc.test_static_entry_allocates_nothing(world[1], world[2], orc, gen)
