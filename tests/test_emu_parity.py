@@ -1,5 +1,4 @@
-"""The gpu-marked parity tests, all but the two that need streams or host threads side by side, run
-as they are (tests/test_gpu_parity.py, the same functions) with the library built for the host
+"""The gpu-marked parity tests run as they are (tests/test_gpu_parity.py, the same functions) with the library built for the host
 (libhomcomp_emu.so, tests/emu) behind the same binding and helper: crafted streams of every plane
 count, mode and outlier width, the bit-plane paths, payloads of random bytes under valid headers,
 zero blocks, special values, empty input, truncated sizes, unaligned stream pointers, ragged
@@ -172,3 +171,14 @@ def test_static_entry_in_a_graph(world, orc, gen):
 
 def test_static_entry_allocates_nothing(world, orc, gen):
     no_alloc.test_static_entry_allocates_nothing(world[1], world[2], orc, gen)
+
+
+# ---- several callers at once: on the model every launch runs alone, whichever host thread makes it, so
+#      what these two exercise here is the library's host side (its locks, the per-device state, the
+#      workspaces created while other threads launch), not the overlap of kernels
+def test_two_streams_do_not_overlap_their_scans(world, orc, gen):
+    parity.test_two_streams_do_not_overlap_their_scans(world[1], world[2], orc, gen)
+
+
+def test_workspaces_created_while_other_threads_launch(world, orc, gen):
+    parity.test_workspaces_created_while_other_threads_launch(world[1], world[2], orc, gen)
