@@ -174,11 +174,8 @@ def test_static_entry_allocates_nothing(world, orc, gen):
 
 
 # ---- several callers at once: on the model every launch runs alone, whichever host thread makes it, so
-#      what these two exercise here is the library's host side (its locks, the per-device state, the
-#      workspaces created while other threads launch), not the overlap of kernels
-def test_two_streams_do_not_overlap_their_scans(world, orc, gen):
-    parity.test_two_streams_do_not_overlap_their_scans(world[1], world[2], orc, gen)
-
-
+#      what this exercises here is the library's host side (its locks, the per-device state, the
+#      workspaces created while other threads launch), not the overlap of kernels.  (The test with two
+#      streams passes on the model too, HOMCOMP_CPU_MODEL=1, but is a minute of sequential calls there.)
 def test_workspaces_created_while_other_threads_launch(world, orc, gen):
     parity.test_workspaces_created_while_other_threads_launch(world[1], world[2], orc, gen)
