@@ -78,6 +78,7 @@ struct emu_wave {
     unsigned arrived, gen;     // of the meeting under way; meetings so far
     unsigned site;             // the place in the program the meeting's first lane came from
     uint64_t slot[2][64];
+    uint64_t present[2];       // the lanes that took part in the meeting whose values the slot array holds
     std::vector<emu_store> log;
     void *main_sp;             // the wave thread's own stack pointer while its lanes run
     const uint8_t *stacks;     // the lanes' stacks, one after the other, stack_bytes each
@@ -194,8 +195,16 @@ inline void emu_release(emu_wave *w)
     w->arrived = 0;
     w->gen++;
 }
+// (for a meeting with values: who is there, noted by the lane that arrives last)
+inline void emu_note_present(emu_wave *w, unsigned p)
+{
+    uint64_t m = 0;
+    for (unsigned l = 0; l < w->count; ++l)
+        if (!w->lanes[l].done) m |= 1ull << l;
+    w->present[p] = m;
+}
 // All lanes of the wave that have not left the kernel meet; true in the one that arrived last.
-inline bool emu_meet(unsigned site)
+inline bool emu_meet(unsigned site, int parity = -1)
 {
     emu_wave *w = emu_wave_of_thread;
     if (w->arrived == 0) {
@@ -207,6 +216,7 @@ inline bool emu_meet(unsigned site)
     }
     const unsigned my = w->gen;
     if (++w->arrived == w->live) {
+        if (parity >= 0) emu_note_present(w, (unsigned)parity);
         emu_release(w);
         return true;
     }
@@ -219,16 +229,17 @@ inline uint64_t emu_exchange(unsigned site, uint64_t mine, int src)
     emu_wave *w = emu_wave_of_thread;
     const unsigned p = emu_cur->parity++ & 1u;
     w->slot[p][emu_lane] = mine;
-    emu_meet(site);
+    emu_meet(site, (int)p);
     return src >= 0 ? w->slot[p][src] : 0;
 }
-// the same, every lane seeing all values (valid until the lane's next meeting but one)
-inline const uint64_t *emu_gather(unsigned site, uint64_t mine)
+// the same, every lane seeing all values (valid until the lane's next meeting but one); `present`: who took part
+inline const uint64_t *emu_gather(unsigned site, uint64_t mine, uint64_t *present)
 {
     emu_wave *w = emu_wave_of_thread;
     const unsigned p = emu_cur->parity++ & 1u;
     w->slot[p][emu_lane] = mine;
-    emu_meet(site);
+    emu_meet(site, (int)p);
+    *present = w->present[p];
     return w->slot[p];
 }
 
@@ -277,11 +288,11 @@ inline int emu_readfirstlane(unsigned site, int v)
 inline int emu_readlane(unsigned site, int v, int lane) { return (int)(uint32_t)emu_exchange(site, (uint32_t)v, lane & 63); }
 inline uint64_t emu_ballot(unsigned site, bool pred)
 {
-    const uint64_t *all = emu_gather(site, pred ? 1u : 0u);
-    const emu_wave *w = emu_wave_of_thread;
+    uint64_t present = 0;
+    const uint64_t *all = emu_gather(site, pred ? 1u : 0u, &present);
     uint64_t m = 0;
-    for (unsigned l = 0; l < w->count; ++l)
-        if (!w->lanes[l].done) m |= (all[l] & 1u) << l;
+    for (unsigned l = 0; l < 64; ++l)
+        if ((present >> l) & 1u) m |= (all[l] & 1u) << l;
     return m;
 }
 template <typename T>

@@ -105,7 +105,11 @@ extern "C" inline void emu_lane_entry()
     if (w->live == 0) {
         emu_switch_stacks(&me->sp, w->main_sp, w->main_stack, w->main_stack_bytes, true);   // the wave is through; does not come back
     }
-    if (w->arrived == w->live) emu_release(w);   // the others were waiting for this lane only
+    if (w->arrived == w->live) {                 // the others were waiting for this lane only
+        emu_note_present(w, 0);
+        emu_note_present(w, 1);
+        emu_release(w);
+    }
     emu_next_lane(w);                             // does not come back either
     abort();
 }

@@ -113,6 +113,21 @@ def build(force: bool = False) -> str:
     return BINARY
 
 
+SELFTEST = os.path.join(GEN, "model_selftest")
+
+
+def build_selftest(force: bool = False) -> str:
+    """The execution model checked against itself (model_selftest.cpp); returns the program's path."""
+    import subprocess
+
+    src = os.path.join(HERE, "model_selftest.cpp")
+    deps = [src] + [os.path.join(HERE, f) for f in ("amdgcn_emu.hpp", "emu_runtime.hpp")]
+    if force or not os.path.exists(SELFTEST) or any(os.path.getmtime(f) > os.path.getmtime(SELFTEST) for f in deps):
+        os.makedirs(GEN, exist_ok=True)
+        subprocess.run([CLANG, *CXXFLAGS, "-I" + HERE, "-o", SELFTEST, src], check=True)
+    return SELFTEST
+
+
 def build_library(force: bool = False) -> str:
     """The whole library (C ABI, workspace logic, launchers, kernels) built for the host against the
     execution model: libhomcomp_emu.so exports what libhomcomp_amd.so exports, plus the model's
@@ -165,3 +180,4 @@ if __name__ == "__main__":
     print(build(force=True))
     print(build_library(force=True))
     print(build_programs(force=True))
+    print(build_selftest(force=True))
