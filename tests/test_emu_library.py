@@ -228,6 +228,34 @@ def test_bounded_wait_reported_once_then_recovery(dev, orc, gen):
         same(out[:L].numpy(), want, "after the recovery")
 
 
+def test_a_grid_that_is_not_resident_ends_with_an_error(dev, orc, gen, monkeypatch):
+    """The condition the bounded waits exist for, for real: the device holds fewer workgroups at a
+    time than the launch has (EMU_RESIDENT), so the data workgroups that run first wait for a scan
+    server that cannot start before they end.  Every wave gives up at its bound, the kernels run to
+    their end, the call is reported as failed, nothing is written outside the output buffer (it ends
+    at an inaccessible page), and on a device that holds the grid the same workspace works again."""
+    binding, t = dev
+    n = 6 * 32768
+    x = gen.smooth_np(n, 131)
+    eb = np.float32(8e-4)
+    want = orc.compress(x, eb)
+    dx = t.from_numpy(x).cuda()
+    out = t.full((binding.max_stream_bytes(n),), 0xC3, dtype=t.uint8, device="cuda")
+    with binding.Workspace(n) as ws:
+        ws.set_option(binding.OPT_SPIN_LIMIT, 50)
+        monkeypatch.setenv("EMU_RESIDENT", "2")
+        ws.compress(dx, float(eb), out)
+        with pytest.raises(binding.HomCompError) as info:
+            ws.last_size()
+        assert info.value.status == binding.ERR_SCAN_TIMEOUT
+        ws.last_size()                               # reported once
+        monkeypatch.delenv("EMU_RESIDENT")
+        ws.set_option(binding.OPT_SPIN_LIMIT, 1 << 16)
+        ws.compress(dx, float(eb), out)
+        L = ws.last_size()
+        same(out[:L].numpy(), want, "on a device that holds the grid")
+
+
 def test_epoch_wrap(dev, orc, gen, monkeypatch):
     """The scan words carry a 22-bit epoch; a workspace started just below the last eager epoch
     crosses the wrap (the tagged words are cleared there) and goes on giving the oracle's bytes."""
