@@ -18,6 +18,7 @@
 #pragma once
 
 #include <signal.h>
+#include <stdio_ext.h>
 #include <sys/mman.h>
 #include <sys/prctl.h>
 #include <sys/wait.h>
@@ -217,6 +218,7 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
     const unsigned n = grid.x * grid.y * grid.z, limit = emu_resident_limit(), workers = n < limit ? n : limit;
     pid_t *kids = new pid_t[workers];
     const pid_t parent = getpid();
+    if (getenv("EMU_TRACE")) fprintf(stderr, "EMU: a grid of %u workgroups of %u lanes, %u at a time\n", n, block.x, workers);
     unsigned started = 0;
     bool ok = true;
     fflush(nullptr);
@@ -231,9 +233,14 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
             // a worker does not outlive the program that launched it (one that was killed at a time limit, say)
             prctl(PR_SET_PDEATHSIG, SIGKILL);
             if (getppid() != parent) _exit(6);
+            // The worker inherits a copy of every stdio buffer as it was at the fork, with whatever another
+            // host thread had in it at that moment (the unwritten end of a file, half a line): none of that
+            // is the worker's to write.  What the program's standard output held is dropped, the other
+            // streams are never flushed here (_exit), and only what the kernel itself prints goes out.
+            __fpurge(stdout);
             emu_worker w{&kernel, block.x, i, workers, n, grid.x};
             emu_run_worker(w);
-            fflush(nullptr);
+            fflush(stdout);
             _exit(0);
         }
         kids[started++] = k;

@@ -9,11 +9,15 @@
 //   model_selftest beyond_buffer  a descriptor over memory no allocation holds: reported
 //   model_selftest beyond_lds     a store behind the dynamic LDS the launch asked for: reported
 //   model_selftest guard_page     a plain store one byte behind an allocation: a fault of the workgroup
+//   model_selftest host_threads FILE   launches from one host thread while another writes FILE through
+//                                 stdio: the workgroups' processes add nothing to it, a kernel's printf arrives once
 #define EMU_DYN_LDS 4096
 #define EMU_DEFINE_GLOBALS
 #include "hip/hip_runtime.h"
 
+#include <atomic>
 #include <string>
+#include <thread>
 
 namespace {
 
@@ -98,6 +102,14 @@ __global__ void k_guard_page(uint8_t *buf, size_t bytes)
     if (threadIdx.x == 0) buf[bytes] = 1;
 }
 
+__global__ void k_says_hello(uint32_t *count)
+{
+    if (threadIdx.x == 0) {
+        count[blockIdx.x] += 1;
+        if (blockIdx.x == 0 && count[0] == 1) printf("a kernel's line\n");
+    }
+}
+
 int fail(const char *what)
 {
     fprintf(stderr, "model_selftest: %s\n", what);
@@ -154,12 +166,42 @@ int semantics()
     return 0;
 }
 
+// A workgroup is a forked process: it starts with a copy of every stdio buffer of the program, as
+// another host thread had filled it at that moment, and must not write any of that out.
+int host_threads(const char *path)
+{
+    FILE *f = fopen(path, "wb");
+    if (!f) return fail("the file");
+    std::atomic<bool> stop{false};
+    size_t records = 0;
+    std::thread writer([&]() {
+        char record[100];
+        while (!stop.load()) {
+            memset(record, 'a' + (int)(records % 26), sizeof(record));
+            fwrite(record, 1, sizeof(record), f);     // stays in the stream's buffer most of the time
+            ++records;
+            usleep(20);
+        }
+    });
+    uint32_t *count = (uint32_t *)emu_device_alloc_named(2 * sizeof(uint32_t), "count");
+    count[0] = count[1] = 0;
+    for (int i = 0; i < 150; ++i) hipLaunchKernelGGL(k_says_hello, dim3(2), dim3(64), 0, 0, count);
+    stop.store(true);
+    writer.join();
+    fclose(f);
+    if (hipGetLastError() != hipSuccess) return fail("a launch");
+    if (count[0] != 150 || count[1] != 150) return fail("the launches' count");
+    printf("records %zu\n", records);
+    return 0;
+}
+
 }  // namespace
 
 int main(int argc, char **argv)
 {
     const std::string what = argc > 1 ? argv[1] : "";
     if (what == "semantics") return semantics();
+    if (what == "host_threads" && argc > 2) return host_threads(argv[2]);
     Out *out = (Out *)emu_device_alloc_named(sizeof(Out), "out");
     if (what == "divergent") {
         hipLaunchKernelGGL(k_divergent, dim3(1), dim3(64), 0, 0, out);
@@ -172,7 +214,7 @@ int main(int argc, char **argv)
         uint8_t *buf = (uint8_t *)emu_device_alloc_named(100, "buf", 1);
         hipLaunchKernelGGL(k_guard_page, dim3(1), dim3(64), 0, 0, buf, (size_t)100);
     } else {
-        fprintf(stderr, "usage: %s semantics|divergent|beyond_buffer|beyond_lds|guard_page\n", argv[0]);
+        fprintf(stderr, "usage: %s semantics|divergent|beyond_buffer|beyond_lds|guard_page|host_threads FILE\n", argv[0]);
         return 2;
     }
     // the kernels above must not get away with it

@@ -230,8 +230,9 @@ def test_bounded_wait_reported_once_then_recovery(dev, orc, gen):
 
 def test_a_grid_that_is_not_resident_ends_with_an_error(dev, orc, gen, monkeypatch):
     """The condition the bounded waits exist for, for real: the device holds fewer workgroups at a
-    time than the launch has (EMU_RESIDENT), so the data workgroups that run first wait for a scan
-    server that cannot start before they end.  Every wave gives up at its bound, the kernels run to
+    time than the launch has (EMU_RESIDENT: one, where the launch is a data workgroup and the scan
+    server behind it), so the data waves wait for a scan server that cannot start before they end
+    (with room for both, the wait's outcome would hang on which process starts faster).  Every wave gives up at its bound, the kernels run to
     their end, the call is reported as failed, nothing is written outside the output buffer (it ends
     at an inaccessible page), and on a device that holds the grid the same workspace works again."""
     binding, t = dev
@@ -243,7 +244,7 @@ def test_a_grid_that_is_not_resident_ends_with_an_error(dev, orc, gen, monkeypat
     out = t.full((binding.max_stream_bytes(n),), 0xC3, dtype=t.uint8, device="cuda")
     with binding.Workspace(n) as ws:
         ws.set_option(binding.OPT_SPIN_LIMIT, 50)
-        monkeypatch.setenv("EMU_RESIDENT", "2")
+        monkeypatch.setenv("EMU_RESIDENT", "1")
         ws.compress(dx, float(eb), out)
         with pytest.raises(binding.HomCompError) as info:
             ws.last_size()

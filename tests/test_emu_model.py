@@ -31,3 +31,18 @@ def test_what_the_model_must_catch(selftest, case, report):
     r = run(selftest, case)
     assert r.returncode == 3 and "launch failed" in r.stdout, r.stdout + r.stderr
     assert report in r.stderr, r.stderr
+
+
+def test_workgroup_processes_write_nothing_of_the_host_threads(selftest, tmp_path):
+    """A workgroup is a forked process and starts with a copy of every stdio buffer of the program.
+    One host thread launches kernels while another writes a file in small records: the file holds
+    exactly those records (no buffered end written twice), and a line a kernel prints arrives once."""
+    path = tmp_path / "records"
+    r = subprocess.run([selftest, "host_threads", str(path)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("a kernel's line") == 1, r.stdout
+    records = int(r.stdout.split("records ")[1].split()[0])
+    data = path.read_bytes()
+    assert len(data) == 100 * records
+    want = b"".join(bytes([ord("a") + i % 26]) * 100 for i in range(records))
+    assert data == want
