@@ -222,6 +222,9 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
     unsigned started = 0;
     bool ok = true;
     fflush(nullptr);
+    // the workers check accesses against the list of buffers as it is when they start: no other host
+    // thread is half-way through changing it then (the workers never take this lock themselves)
+    pthread_mutex_lock(&emu_alloc_lock);
     for (unsigned i = 0; i < workers; ++i) {
         const pid_t k = fork();
         if (k < 0) {
@@ -245,6 +248,7 @@ inline bool emu_run_grid(const std::function<void()> &kernel, emu_dim3 grid, emu
         }
         kids[started++] = k;
     }
+    pthread_mutex_unlock(&emu_alloc_lock);
     for (unsigned i = 0; i < started; ++i) {
         int status = 0;
         waitpid(kids[i], &status, 0);
