@@ -199,6 +199,7 @@ int main(int argc, char **argv)
     p.recip = 0.5f / eb;
     p.epoch = 7;
     p.spin_limit = 1u << 30;
+    if (const char *e = getenv("EMU_SPIN_LIMIT")) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);   // looks a wait may take (a test of the bounded waits)
     p.out_slots = slots;
     p.sliced = kind;
     p.plain = plain;

@@ -28,7 +28,7 @@ class Emu:
         self.binary, self.tmp, self.calls = binary, tmp, 0
 
     def run(self, op, n, eb, a, b=None, groups=2, budget=BUDGETS[2], kind=0, slots=2, plain=0, dtype=np.uint8, offsets=False,
-            stated_a=None):
+            stated_a=None, env=None, expect=0):
         self.calls += 1
         pa, pb, po, pf = (os.path.join(self.tmp, x) for x in ("a", "b", "out", "ofs"))
         for path, data in ((pa, a), (pb, b)):
@@ -38,8 +38,10 @@ class Emu:
                 pa if a is not None else "-", pb if b is not None else "-", po, pf if offsets else "-"]
         if stated_a is not None:
             args.append(str(stated_a))
-        r = subprocess.run(args, capture_output=True, text=True, timeout=600)
-        assert r.returncode == 0, f"{' '.join(args[1:9])}: exit {r.returncode}\n{r.stderr[-3000:]}"
+        r = subprocess.run(args, capture_output=True, text=True, timeout=600, env=dict(os.environ, **(env or {})))
+        assert r.returncode == expect, f"{' '.join(args[1:9])}: exit {r.returncode}\n{r.stderr[-3000:]}"
+        if expect:
+            return r.stderr
         out = np.fromfile(po, dtype=dtype)
         return (out, np.fromfile(pf, dtype=np.uint64)) if offsets else out
 
@@ -242,3 +244,20 @@ def test_quant_predict_and_value_range(emu, orc, gen):
         lo, hi = orc.value_range(x)
         got = emu.run("value_range", n, eb, x, groups=3, dtype=np.float32)
         assert got[0] == lo and got[1] == hi, f"value_range n={n}"
+
+
+@pytest.mark.parametrize("op", ["compress", "hom_sum_f32"])
+def test_a_grid_larger_than_the_device_holds(emu, orc, gen, op):
+    """Six data workgroups and the scan server behind them on a device that holds three workgroups
+    at a time: the first three wait for a server that cannot start before two of them have ended.
+    Every wait ends at its bound, every workgroup runs to its end without touching memory that is
+    not its own (any such access ends the run with another status), and the error word is raised;
+    the same launch on a device that holds it gives the oracle's bytes."""
+    n = 48 * 4096 + 77
+    x, y = gen.smooth_np(n, 7), gen.smooth_np(n, 8)
+    eb = bound_of(orc, 1e-5, x, y)
+    sa = orc.compress(x, eb)
+    a, b, want = (x, None, sa) if op == "compress" else (sa, y, orc.hom_sum_f32(sa, y, eb))
+    report = emu.run(op, n, eb, a, b, groups=6, env={"EMU_RESIDENT": "3", "EMU_SPIN_LIMIT": "20"}, expect=5)
+    assert "the kernels raised the error word" in report and "abnormally" not in report, report
+    same(emu.run(op, n, eb, a, b, groups=6, env={"EMU_SPIN_LIMIT": "20000"}), want, "with the whole grid on the device")
