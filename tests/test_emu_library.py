@@ -296,3 +296,75 @@ def test_argument_checks(dev, gen):
         # n = 0: an empty stream
         assert L.homcomp_compress_f32(h, x.data_ptr(), 0, 1e-3, out.data_ptr(), None, None) == 0
         assert ws.last_size() == 0
+
+
+def test_integer_delta_ring_with_lengths_left_on_the_device(dev, orc, gen):
+    """The reduce-scatter of the reference's integer-delta ring (HomComp/src/cuda_awareallreduce.cu:
+    212-235) in the shape in which no length comes back to the host between steps: three ranks as
+    host threads with a workspace each, every step homcomp_quant_predict_f32 into a buffer of
+    max-block ints followed by homcomp_hom_sum_i32 on the buffer that arrived, its size stated as
+    the buffer's capacity (the stream is followed by whatever the buffer held before), blocks of a
+    ragged length, the lengths written to device words only.  Every access the kernels make is
+    checked against the buffers (each ends at an inaccessible page); every step's bytes against the
+    oracle on the very buffer the rank received."""
+    import threading
+    binding, t = dev
+    ranks, block = 3, 4096 * 9 + 77
+    data = [gen.smooth_np(ranks * block, 140 + r) * np.float32(1.0 + r) for r in range(ranks)]
+    eb = np.float32(2e-4)
+    cap = binding.max_stream_bytes(block)
+    room = cap + binding.STREAM_SLACK
+    # two buffers per rank (a step reads one and writes the other), filled with what "earlier use" left
+    bufs = [[t.full((room,), 0x3C + 16 * r + i, dtype=t.uint8, device="cuda") for i in range(2)] for r in range(ranks)]
+    inbox = [t.full((room,), 0x77, dtype=t.uint8, device="cuda") for _ in range(ranks)]
+    quant = [t.full((block + 31,), 424242, dtype=t.int32, device="cuda") for _ in range(ranks)]
+    lengths = [t.zeros((ranks,), dtype=t.int64, device="cuda") for _ in range(ranks)]
+    local = [[t.from_numpy(np.ascontiguousarray(data[r][b * block:(b + 1) * block])).cuda() for b in range(ranks)] for r in range(ranks)]
+    received = [[None] * (ranks - 1) for _ in range(ranks)]    # host copies of what arrived, for the oracle
+    produced = [[None] * ranks for _ in range(ranks)]
+    gate = threading.Barrier(ranks)
+    errors = []
+
+    def rank_main(r):
+        try:
+            with binding.Workspace(block) as ws:
+                cur = 0
+                ws.compress(local[r][r], float(eb), bufs[r][cur], stream_len=lengths[r][0:1])
+                produced[r][0] = bufs[r][cur].numpy().copy()
+                for step in range(ranks - 1):
+                    gate.wait()
+                    inbox[(r + 1) % ranks].copy_(bufs[r][cur])          # the send: the whole buffer, no length known
+                    gate.wait()
+                    received[r][step] = inbox[r].numpy().copy()
+                    b = (r - 1 - step) % ranks
+                    binding.quant_predict(local[r][b], float(eb), quant[r], n=block)
+                    cur ^= 1
+                    ws.hom_sum_i32(inbox[r], cap, quant[r], bufs[r][cur], stream_len=lengths[r][step + 1:step + 2], n=block)
+                    produced[r][step + 1] = bufs[r][cur].numpy().copy()
+                ws.last_size()                                             # the only read-back: no time-out was recorded
+        except Exception as e:  # noqa: BLE001
+            errors.append((r, e))
+            gate.abort()
+
+    threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(ranks)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=600)
+    assert not errors, errors
+    for r in range(ranks):
+        want = orc.compress(data[r][r * block:(r + 1) * block], eb)
+        same(produced[r][0][:want.size], want, f"rank {r} compress")
+        assert int(lengths[r][0]) == want.size
+        for step in range(ranks - 1):
+            b = (r - 1 - step) % ranks
+            deltas = orc.quant_predict(data[r][b * block:(b + 1) * block], eb)
+            want = orc.hom_sum_i32(received[r][step][:cap], deltas, cmp_in_size=cap)
+            same(produced[r][step + 1][:want.size], want, f"rank {r} step {step}")
+            assert int(lengths[r][step + 1]) == want.size, f"rank {r} step {step}: the length on the device"
+    # the sums themselves: block (r + 1) % ranks at rank r holds every rank's contribution
+    for r in range(ranks):
+        b = (r + 1) % ranks
+        q = sum(orc.quantize_array(data[k][b * block:(b + 1) * block], eb).astype(np.int64) for k in range(ranks))
+        length = int(lengths[r][ranks - 1])
+        assert np.array_equal(orc.decode_quants(produced[r][ranks - 1][:length], block).astype(np.int64), q), f"block {b}"
