@@ -86,6 +86,8 @@ struct emu_wave {
     const void *main_stack;    // the wave thread's own stack (known to a sanitizer build only)
     size_t main_stack_bytes;
     const void *kernel;        // std::function<void()> of the launch
+    uint8_t *guards[8];        // behind the LDS slots this wave has used in the workgroup under way (emu_stage_slot)
+    unsigned n_guards;
 };
 extern thread_local emu_wave *emu_wave_of_thread;
 extern thread_local emu_lane_ctx *emu_cur;   // the lane that is running on this thread
@@ -96,11 +98,32 @@ extern pthread_barrier_t emu_block_barrier;   // of the workgroup's wave threads
 // the size of the launch under way holds a pattern that must still be there when a workgroup ends.
 extern uint8_t *emu_dynamic_lds;          // where the running kernel's array is (a kernel with one says so)
 extern size_t emu_dynamic_lds_bytes;      // of the launch under way
-inline void emu_note_dynamic_lds(uint8_t *array)
+extern size_t emu_dynamic_lds_extra;      // bytes the model adds between the parts of the array (emu_stage_slot); the array is that much longer
+inline void emu_note_dynamic_lds(uint8_t *array, size_t extra = 0)
 {
     // the first lane of the workgroup to come by lays the pattern (nothing has used the array yet)
-    if (__sync_bool_compare_and_swap(&emu_dynamic_lds, (uint8_t *)nullptr, array))
-        memset(array + emu_dynamic_lds_bytes, 0xD5, EMU_DYN_LDS - emu_dynamic_lds_bytes);
+    if (__sync_bool_compare_and_swap(&emu_dynamic_lds, (uint8_t *)nullptr, array)) {
+        emu_dynamic_lds_extra = extra;
+        memset(array + emu_dynamic_lds_bytes + extra, 0xD5, EMU_DYN_LDS - emu_dynamic_lds_bytes);
+    }
+}
+// A kernel that cuts its dynamic LDS into slots (`slots` per wave, `slot_bytes` each) gets them with
+// EMU_SLOT_GUARD bytes of pattern behind each, which must be intact when the workgroup ends: a
+// wave that writes beyond a slot is found, not just one that writes beyond the whole array.
+#define EMU_SLOT_GUARD 256
+inline uint8_t *emu_stage_slot(uint8_t *array, uint32_t wave, uint32_t slot, uint32_t slots, uint32_t slot_bytes)
+{
+    uint8_t *at = array + (size_t)(wave * slots + slot) * ((size_t)slot_bytes + EMU_SLOT_GUARD);
+    emu_wave *w = emu_wave_of_thread;
+    for (unsigned i = 0; i < w->n_guards; ++i)
+        if (w->guards[i] == at + slot_bytes) return at;
+    if (w->n_guards == sizeof w->guards / sizeof w->guards[0]) {
+        fprintf(stderr, "EMU: a wave with more LDS slots than the model keeps track of\n");
+        abort();
+    }
+    memset(at + slot_bytes, 0xD6, EMU_SLOT_GUARD);   // the wave's first use of the slot: nothing is in it yet
+    w->guards[w->n_guards++] = at + slot_bytes;
+    return at;
 }
 
 // Every access a kernel makes to "device memory" must fall into a registered allocation; the

@@ -156,21 +156,36 @@ inline void *emu_wave_main(void *arg)
         w->arrived = 0;
         w->gen = 0;
         w->log.clear();
+        w->n_guards = 0;
         if (s->index == 0) emu_dynamic_lds = nullptr;
         pthread_barrier_wait(&emu_block_barrier);
         emu_cur = &w->lanes[0];
         w->main_stack = nullptr;
         emu_switch_stacks(&w->main_sp, w->lanes[0].sp, stacks, emu_lane_stack);   // back here when the wave's last lane has left the kernel
         pthread_barrier_wait(&emu_block_barrier);
+        // nothing was written behind an LDS slot of this wave, by any wave (the pattern emu_stage_slot laid)
+        for (unsigned g = 0; g < w->n_guards; ++g)
+            for (unsigned b = 0; b < EMU_SLOT_GUARD; ++b)
+                if (w->guards[g][b] != 0xD6u) {
+                    fprintf(stderr, "EMU: block %u wrote beyond an LDS slot of wave %u (byte %u behind the slot's end)\n", i, s->index, b);
+                    if (getenv("EMU_TRACE")) {
+                        fprintf(stderr, "EMU: slot guard %u of the wave, at %p:", g, (void *)w->guards[g]);
+                        for (unsigned k = 0; k < 48; ++k) fprintf(stderr, " %02x", w->guards[g][k]);
+                        fprintf(stderr, "\n");
+                    }
+                    _exit(5);
+                }
         if (s->index == 0 && emu_dynamic_lds) {
             // nothing was written beyond the dynamic LDS the launch asked for (the pattern emu_note_dynamic_lds laid)
-            for (uint8_t *b = emu_dynamic_lds + emu_dynamic_lds_bytes; b != emu_dynamic_lds + EMU_DYN_LDS; ++b)
+            uint8_t *const end = emu_dynamic_lds + emu_dynamic_lds_bytes + emu_dynamic_lds_extra;
+            for (uint8_t *b = end; b != emu_dynamic_lds + EMU_DYN_LDS + emu_dynamic_lds_extra; ++b)
                 if (*b != 0xD5u) {
                     fprintf(stderr, "EMU: block %u wrote %zu bytes beyond its %zu bytes of dynamic LDS\n", i,
-                            (size_t)(b - emu_dynamic_lds) - emu_dynamic_lds_bytes + 1, emu_dynamic_lds_bytes);
+                            (size_t)(b - end) + 1, emu_dynamic_lds_bytes);
                     _exit(5);
                 }
         }
+        pthread_barrier_wait(&emu_block_barrier);   // the next workgroup's LDS pattern is laid when every wave has looked at its guards
     }
     munmap(stacks, 64 * emu_lane_stack);
     delete w;
@@ -458,6 +473,7 @@ thread_local emu_lane_ctx *emu_cur = nullptr;
 pthread_barrier_t emu_block_barrier;
 uint8_t *emu_dynamic_lds = nullptr;
 size_t emu_dynamic_lds_bytes = 0;
+size_t emu_dynamic_lds_extra = 0;
 emu_graph *emu_capturing = nullptr;
 unsigned long long emu_capture_id = 0;
 emu_alloc emu_allocs[8192];

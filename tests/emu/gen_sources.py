@@ -37,7 +37,11 @@ DEVICE_EDITS = [
     ("        if (w <= o.F) store_u32_any(at + 4u * w, o.w[w]);", "        if (w <= o.F) emu_ordered_store32(at + 4u * w, o.w[w], kWideChunks + 1 + w);"),
 ]
 KERNEL_EDITS = [
-    ("    extern __shared__ __align__(16) uint8_t s_dyn[];", "    static __attribute__((aligned(16), section(\"emu_lds\"))) uint8_t s_dyn[EMU_DYN_LDS];\n    emu_note_dynamic_lds(s_dyn);"),
+    # four waves of up to four slots each, every slot followed by a guard (emu_stage_slot)
+    ("    extern __shared__ __align__(16) uint8_t s_dyn[];",
+     "    static __attribute__((aligned(16), section(\"emu_lds\"))) uint8_t s_dyn[EMU_DYN_LDS + 16 * EMU_SLOT_GUARD];\n    emu_note_dynamic_lds(s_dyn, 16 * EMU_SLOT_GUARD);"),
+    ("        uint8_t *stage = s_dyn + (uint32_t)wave * p.stage_bytes + (uint32_t)obuf * slot_bytes;",
+     "        uint8_t *stage = kEnc ? emu_stage_slot(s_dyn, (uint32_t)wave, (uint32_t)obuf, (uint32_t)D, slot_bytes) : s_dyn;   // (a decoder has no stage)"),
     ('            if constexpr (kSlicedLocal) asm volatile("" : "+v"(fresh_lane));', ""),
     # A wave's LDS instructions take effect in the order of the program, for all its lanes: what the lanes packed is
     # in the stage when the instructions that move it elsewhere read it.  Lanes that are threads have to meet for that.

@@ -8,6 +8,7 @@
 //   model_selftest divergent      a cross-lane operation under a branch that is not uniform: reported
 //   model_selftest beyond_buffer  a descriptor over memory no allocation holds: reported
 //   model_selftest beyond_lds     a store behind the dynamic LDS the launch asked for: reported
+//   model_selftest beyond_slot    a store behind one of the slots a kernel cuts its dynamic LDS into: reported
 //   model_selftest guard_page     a plain store one byte behind an allocation: a fault of the workgroup
 //   model_selftest host_threads FILE   launches from one host thread while another writes FILE through
 //                                 stdio: the workgroups' processes add nothing to it, a kernel's printf arrives once
@@ -95,6 +96,17 @@ __global__ void k_beyond_lds(int)
     emu_note_dynamic_lds(s_dyn);
     s_dyn[threadIdx.x] = 1;          // within the 64 bytes the launch asked for
     if (threadIdx.x == 5) s_dyn[64] = 1;
+}
+
+__global__ void k_beyond_slot(int)
+{
+    static __attribute__((aligned(16), section("emu_lds"))) uint8_t s_dyn[EMU_DYN_LDS + 16 * EMU_SLOT_GUARD];
+    emu_note_dynamic_lds(s_dyn, 16 * EMU_SLOT_GUARD);
+    // two slots of 64 bytes for the one wave; the first is filled to its last byte, the second one byte further
+    uint8_t *first = emu_stage_slot(s_dyn, 0, 0, 2, 64), *second = emu_stage_slot(s_dyn, 0, 1, 2, 64);
+    first[threadIdx.x] = 1;
+    second[threadIdx.x] = 1;
+    if (threadIdx.x == 9) second[64] = 1;
 }
 
 __global__ void k_guard_page(uint8_t *buf, size_t bytes)
@@ -210,11 +222,13 @@ int main(int argc, char **argv)
         hipLaunchKernelGGL(k_beyond_buffer, dim3(1), dim3(64), 0, 0, stray);
     } else if (what == "beyond_lds") {
         hipLaunchKernelGGL(k_beyond_lds, dim3(1), dim3(64), 64, 0, 0);
+    } else if (what == "beyond_slot") {
+        hipLaunchKernelGGL(k_beyond_slot, dim3(1), dim3(64), 128, 0, 0);
     } else if (what == "guard_page") {
         uint8_t *buf = (uint8_t *)emu_device_alloc_named(100, "buf", 1);
         hipLaunchKernelGGL(k_guard_page, dim3(1), dim3(64), 0, 0, buf, (size_t)100);
     } else {
-        fprintf(stderr, "usage: %s semantics|divergent|beyond_buffer|beyond_lds|guard_page|host_threads FILE\n", argv[0]);
+        fprintf(stderr, "usage: %s semantics|divergent|beyond_buffer|beyond_lds|beyond_slot|guard_page|host_threads FILE\n", argv[0]);
         return 2;
     }
     // the kernels above must not get away with it

@@ -1,5 +1,5 @@
 """The CPU execution model checked against itself (tests/emu/model_selftest.cpp): the cross-lane and
-bit-field operations against their definitions in the instruction set, and the four things the
+bit-field operations against their definitions in the instruction set, and the five things the
 model is there to catch -- each must end the run the way the model promises, or the other
 test_emu_* files prove less than they seem to."""
 import subprocess
@@ -25,6 +25,7 @@ def test_operations_have_their_documented_meaning(selftest):
     ("divergent", "at different places of the program"),
     ("beyond_buffer", "is outside every buffer"),
     ("beyond_lds", "beyond its 64 bytes of dynamic LDS"),
+    ("beyond_slot", "wrote beyond an LDS slot of wave 0 (byte 0 behind the slot's end)"),
     ("guard_page", "segmentation fault, an access beyond a buffer"),
 ])
 def test_what_the_model_must_catch(selftest, case, report):
