@@ -86,7 +86,7 @@ struct emu_wave {
     const void *main_stack;    // the wave thread's own stack (known to a sanitizer build only)
     size_t main_stack_bytes;
     const void *kernel;        // std::function<void()> of the launch
-    uint8_t *guards[8];        // behind the LDS slots this wave has used in the workgroup under way (emu_stage_slot)
+    uint8_t *guards[16];       // behind the parts of LDS that are this wave's own, in the workgroup under way (emu_guard_behind)
     unsigned n_guards;
 };
 extern thread_local emu_wave *emu_wave_of_thread;
@@ -107,22 +107,28 @@ inline void emu_note_dynamic_lds(uint8_t *array, size_t extra = 0)
         memset(array + emu_dynamic_lds_bytes + extra, 0xD5, EMU_DYN_LDS - emu_dynamic_lds_bytes);
     }
 }
-// A kernel that cuts its dynamic LDS into slots (`slots` per wave, `slot_bytes` each) gets them with
-// EMU_SLOT_GUARD bytes of pattern behind each, which must be intact when the workgroup ends: a
-// wave that writes beyond a slot is found, not just one that writes beyond the whole array.
+// Guards inside LDS: EMU_SLOT_GUARD bytes of pattern behind a part of an array that belongs to one
+// wave, laid at the wave's first mention of it and intact when the workgroup ends -- or a wave
+// has written beyond its part, which the end of the whole array would not show.
 #define EMU_SLOT_GUARD 256
+inline void emu_guard_behind(uint8_t *end_of_part)
+{
+    emu_wave *w = emu_wave_of_thread;
+    for (unsigned i = 0; i < w->n_guards; ++i)
+        if (w->guards[i] == end_of_part) return;
+    if (w->n_guards == sizeof w->guards / sizeof w->guards[0]) {
+        fprintf(stderr, "EMU: a wave with more guarded parts of LDS than the model keeps track of\n");
+        abort();
+    }
+    memset(end_of_part, 0xD6, EMU_SLOT_GUARD);   // the wave's first mention of the part: nothing is in it yet
+    w->guards[w->n_guards++] = end_of_part;
+}
+// A kernel that cuts its dynamic LDS into slots (`slots` per wave, `slot_bytes` each) gets them
+// with a guard behind each.
 inline uint8_t *emu_stage_slot(uint8_t *array, uint32_t wave, uint32_t slot, uint32_t slots, uint32_t slot_bytes)
 {
     uint8_t *at = array + (size_t)(wave * slots + slot) * ((size_t)slot_bytes + EMU_SLOT_GUARD);
-    emu_wave *w = emu_wave_of_thread;
-    for (unsigned i = 0; i < w->n_guards; ++i)
-        if (w->guards[i] == at + slot_bytes) return at;
-    if (w->n_guards == sizeof w->guards / sizeof w->guards[0]) {
-        fprintf(stderr, "EMU: a wave with more LDS slots than the model keeps track of\n");
-        abort();
-    }
-    memset(at + slot_bytes, 0xD6, EMU_SLOT_GUARD);   // the wave's first use of the slot: nothing is in it yet
-    w->guards[w->n_guards++] = at + slot_bytes;
+    emu_guard_behind(at + slot_bytes);
     return at;
 }
 

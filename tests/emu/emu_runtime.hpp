@@ -163,13 +163,13 @@ inline void *emu_wave_main(void *arg)
         w->main_stack = nullptr;
         emu_switch_stacks(&w->main_sp, w->lanes[0].sp, stacks, emu_lane_stack);   // back here when the wave's last lane has left the kernel
         pthread_barrier_wait(&emu_block_barrier);
-        // nothing was written behind an LDS slot of this wave, by any wave (the pattern emu_stage_slot laid)
+        // nothing was written behind a part of LDS that is this wave's own, by any wave (the pattern emu_guard_behind laid)
         for (unsigned g = 0; g < w->n_guards; ++g)
             for (unsigned b = 0; b < EMU_SLOT_GUARD; ++b)
                 if (w->guards[g][b] != 0xD6u) {
-                    fprintf(stderr, "EMU: block %u wrote beyond an LDS slot of wave %u (byte %u behind the slot's end)\n", i, s->index, b);
+                    fprintf(stderr, "EMU: block %u wrote beyond a part of LDS of wave %u (byte %u behind its end)\n", i, s->index, b);
                     if (getenv("EMU_TRACE")) {
-                        fprintf(stderr, "EMU: slot guard %u of the wave, at %p:", g, (void *)w->guards[g]);
+                        fprintf(stderr, "EMU: guard %u of the wave, at %p:", g, (void *)w->guards[g]);
                         for (unsigned k = 0; k < 48; ++k) fprintf(stderr, " %02x", w->guards[g][k]);
                         fprintf(stderr, "\n");
                     }

@@ -42,6 +42,12 @@ KERNEL_EDITS = [
      "    static __attribute__((aligned(16), section(\"emu_lds\"))) uint8_t s_dyn[EMU_DYN_LDS + 16 * EMU_SLOT_GUARD];\n    emu_note_dynamic_lds(s_dyn, 16 * EMU_SLOT_GUARD);"),
     ("        uint8_t *stage = s_dyn + (uint32_t)wave * p.stage_bytes + (uint32_t)obuf * slot_bytes;",
      "        uint8_t *stage = kEnc ? emu_stage_slot(s_dyn, (uint32_t)wave, (uint32_t)obuf, (uint32_t)D, slot_bytes) : s_dyn;   // (a decoder has no stage)"),
+    # the rows of the static arrays that the code reaches through pointers: a guard behind each wave's row
+    ("    __shared__ __align__(16) uint8_t s_in[kW][NIN > 0 ? kInBytes : 16];", "    __shared__ __align__(16) uint8_t s_in[kW][(NIN > 0 ? kInBytes : 16) + EMU_SLOT_GUARD];"),
+    ("    __shared__ __align__(16) float s_tr[kW][kEnc ? 4 : 512]; ", "    __shared__ __align__(16) float s_tr[kW][(kEnc ? 4 : 512) + EMU_SLOT_GUARD / 4]; "),
+    ("    const int lane = threadIdx.x & 63;\n    const int k = lane & 3;\n    const int quad = lane >> 2;\n    // tile indices are 32-bit",
+     "    const int lane = threadIdx.x & 63;\n    emu_guard_behind(&s_in[wave][NIN > 0 ? kInBytes : 16]);\n    emu_guard_behind((uint8_t *)&s_tr[wave][kEnc ? 4 : 512]);\n"
+     "    const int k = lane & 3;\n    const int quad = lane >> 2;\n    // tile indices are 32-bit"),
     ('            if constexpr (kSlicedLocal) asm volatile("" : "+v"(fresh_lane));', ""),
     # A wave's LDS instructions take effect in the order of the program, for all its lanes: what the lanes packed is
     # in the stage when the instructions that move it elsewhere read it.  Lanes that are threads have to meet for that.

@@ -25,7 +25,7 @@ def test_operations_have_their_documented_meaning(selftest):
     ("divergent", "at different places of the program"),
     ("beyond_buffer", "is outside every buffer"),
     ("beyond_lds", "beyond its 64 bytes of dynamic LDS"),
-    ("beyond_slot", "wrote beyond an LDS slot of wave 0 (byte 0 behind the slot's end)"),
+    ("beyond_slot", "wrote beyond a part of LDS of wave 0 (byte 0 behind its end)"),
     ("guard_page", "segmentation fault, an access beyond a buffer"),
 ])
 def test_what_the_model_must_catch(selftest, case, report):
